@@ -1,0 +1,151 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse-mask attention hot path on one MI355X.
+
+A step is one pass of the hot path over one batch of synthetic input, as the reference times it
+(run.py:147-155, :172-183): pack_mask(bool mask) -> allocate out -> fused attention forward, called
+through the `sparse_attn_cuda` module with all inputs already resident in HBM.  The headline
+value is dense-equivalent TFLOP/s, 4*B*H*N*N*D per step whatever the sparsity (run.py:198-203).
+
+Prints ONE JSON line.  Besides the whole-step figure it carries
+  roofline      the fused attention kernel alone (the dominant kernel) against the dense FP16 MFMA
+                peak, from stream-event timing of back-to-back launches on the launch stream;
+  roofline_pack the packer alone against the HBM peak;
+  cpu_baseline  the oracle's PyTorch formulation of the same workload on the host cores.
+"""
+import argparse
+import ctypes
+import importlib
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "sparse-mask-attention_amd")
+for p in (PKG, ROOT):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+# Published figure for exactly this metric and configuration (pack_mask included in the timing):
+# 27.66 dense-equivalent TFLOP/s on an RTX 3080, reference README.md:13.
+PUBLISHED_TFLOPS = {"C2": 27.66}
+
+
+def event_time_ms(fn, warmup, repeat, torch):
+    """Mean ms per call of `repeat` back-to-back calls between two events on the current stream."""
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(repeat):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / repeat
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on ONE GPU; every (b,h) pair is independent, so more "
+                 "GPUs would each take a slice of the batch with no exchange. Use --gpus 1.")
+
+    import torch
+    import harness
+    sa = importlib.import_module("python.sparse_attention")
+    if not sa.HAS_CUDA_EXT:
+        sys.exit(f"bench.py: HIP extension missing ({sa._EXT_ERROR}); run __graft_entry__.build()")
+    import sparse_attn_cuda as ext
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    dev = torch.device("cuda:0")
+
+    w = harness.WORKLOADS[args.workload]
+    q, k, v, mask = harness.make_inputs(w, seed=42)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    scale = 1.0 / (w.D ** 0.5)
+
+    def step():
+        packed = ext.pack_mask(md)
+        out = torch.empty_like(qd)
+        ext.forward(qd, kd, vd, packed, out, None, scale, False)
+        return out
+
+    # ---- whole step: W untimed, K timed, synchronize on both sides ----
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    value = w.dense_flops / (ms_per_step * 1e-3) / 1e12
+
+    # ---- the two kernels on their own: back-to-back launches between stream events ----
+    packed = ext.pack_mask(md)
+    out = torch.empty_like(qd)
+    reps = max(50, args.steps)
+    attn_ms = event_time_ms(lambda: ext.forward(qd, kd, vd, packed, out, None, scale, False), 10, reps, torch)
+    # the packer through the C ABI into a preallocated buffer (no allocator in the loop)
+    lib = ctypes.CDLL(os.path.join(PKG, "libsma_hip.so"))
+    lib.sma_pack_mask.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
+                                  ctypes.c_int, ctypes.c_void_p]
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    pack_ms = event_time_ms(lambda: lib.sma_pack_mask(md.data_ptr(), packed.data_ptr(), w.B, w.H, w.N, stream),
+                            10, reps, torch)
+    api_ms = event_time_ms(lambda: sa.sparse_attention_func(qd, kd, vd, md), 10, reps, torch)
+
+    attn_tflops = w.dense_flops / (attn_ms * 1e-3) / 1e12
+    pack_gbps = w.pack_bytes / (pack_ms * 1e-3) / 1e9
+    result = {
+        "metric": "dense_equiv_tflops_sparse_attention_fwd_incl_pack_mask",
+        "value": round(value, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": (round(value / PUBLISHED_TFLOPS[w.name], 3) if w.name in PUBLISHED_TFLOPS else None),
+        "dtype": "fp16" if w.dtype == torch.float16 else "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"{w.name}: B={w.B} H={w.H} N={w.N} D={w.D} {w.mask_kind} mask keep_p={w.keep_prob}",
+                   "step": "pack_mask + torch.empty_like + fused forward via sparse_attn_cuda (no LSE)",
+                   "dense_equiv_flop_per_step": w.dense_flops},
+        "attn_kernel_ms": round(attn_ms, 5),
+        "attn_kernel_tflops": round(attn_tflops, 2),
+        "attn_kernel_hbm_gbps": round(w.attn_bytes / (attn_ms * 1e-3) / 1e9, 1),
+        "pack_kernel_ms": round(pack_ms, 5),
+        "api_sparse_attention_func_ms": round(api_ms, 5),
+        "roofline": {"kernel": "attn_fwd_kernel", "bound": "mfma", "achieved": round(attn_tflops, 2),
+                     "peak": harness.MI355X_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(attn_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4), "traffic": None},
+        "roofline_pack": {"kernel": "pack_flat_kernel" if w.N % 32 == 0 else "pack_rows_kernel",
+                          "bound": "hbm", "achieved": round(pack_gbps, 1), "peak": harness.MI355X_HBM_GBPS,
+                          "unit": "GB/s", "frac": round(pack_gbps / harness.MI355X_HBM_GBPS, 4), "traffic": None},
+    }
+
+    if not args.no_cpu_baseline:
+        from oracle import sma_oracle
+        threads = torch.get_num_threads()
+        sec = sma_oracle.time_cpu_reference(q.float(), k.float(), v.float(), mask, reps=3)
+        result["cpu_baseline"] = {
+            "value": round(w.dense_flops / sec / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
+            "kind": "port", "ms": round(sec * 1e3, 2),
+            "sample": f"whole {w.name} workload, fp32 PyTorch formulation of the oracle on the host CPU, "
+                      f"median of 3 after 1 warm-up, torch threads={threads}, os.cpu_count()={os.cpu_count()}"}
+    print(json.dumps(result), flush=True)
+
+
+if __name__ == "__main__":
+    main()

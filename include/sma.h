@@ -1,0 +1,76 @@
+/* sma.h - C ABI of libsma_hip.so: sparse-mask attention for AMD MI355X (gfx950).
+ *
+ * Plain C, plain pointers and sizes.  Every pointer is a DEVICE pointer in the address space of
+ * the GPU that is current on the calling thread; `stream` is a hipStream_t passed as void*
+ * (NULL = the default stream).  All tensors are dense row-major ("contiguous").  Launches are
+ * asynchronous on `stream`; the functions never synchronise, never allocate and keep no state.
+ * Return value: SMA_OK (0) or a negative SMA_ERR_* code; sma_strerror() names it.
+ *
+ * Each entry point cites the interface of the reference implementation that it stands in for
+ * (paths relative to the reference tree).
+ */
+#ifndef SMA_H_
+#define SMA_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SMA_OK                 0
+#define SMA_ERR_NULL_POINTER  -1   /* a required pointer is NULL */
+#define SMA_ERR_BAD_SHAPE     -2   /* a negative extent, or an extent beyond the 32-bit index range */
+#define SMA_ERR_HEAD_DIM      -3   /* head_dim other than 64 */
+#define SMA_ERR_DTYPE         -4   /* dtype other than SMA_DTYPE_F16 / SMA_DTYPE_BF16 */
+#define SMA_ERR_SCALE         -5   /* scale is NaN or infinite */
+#define SMA_ERR_LAUNCH        -6   /* the HIP runtime refused the launch (hipGetLastError) */
+#define SMA_ERR_ALIGNMENT     -7   /* q/k/v/out not 16-byte aligned, or mask_packed/lse not 4-byte aligned */
+
+#define SMA_DTYPE_F16   0
+#define SMA_DTYPE_BF16  1
+
+/* Library version, major*10000 + minor*100 + patch. */
+int sma_version(void);
+
+/* Static, never-NULL description of a return code. */
+const char *sma_strerror(int code);
+
+/* Bit-pack a boolean attend-mask.
+ *
+ *   mask    uint8 [B,H,N,N], one byte per entry, non-zero = attend (torch.bool storage)
+ *   packed  uint32 [B,H,N,ceil(N/32)]; bit j of word w of row i is column 32*w+j of that row;
+ *           bits that stand for columns >= N are written as 0.  Every word is written, so the
+ *           output needs no pre-clearing.
+ *
+ * Replaces: void pack_mask_bits(const bool*, uint32_t*, int B, int H, int N, cudaStream_t)
+ *           csrc/sparse_attention.h:67-72, defined csrc/sparse_attention.cu:603-610
+ *           (kernel pack_mask_kernel, csrc/sparse_attention.cu:549-568).
+ */
+int sma_pack_mask(const uint8_t *mask, uint32_t *packed, int B, int H, int N, void *stream);
+
+/* Fused masked attention forward:  out = softmax_row(mask ? (q k^T) * scale : -inf) v.
+ *
+ *   q, k, v      [B,H,N,D] fp16 or bf16 (dtype), D must be 64
+ *   mask_packed  uint32 [B,H,N,ceil(N/32)] in the sma_pack_mask format (pad bits are ignored)
+ *   out          [B,H,N,D], same dtype; every element is written
+ *   lse          NULL, or float [B,H,N]: natural-log-sum-exp of the kept scaled scores of each
+ *                query row, -inf for a row that keeps no key
+ *   scale        any finite float (the reference passes 1/sqrt(D))
+ *
+ * A query row whose mask keeps no key yields zeros.  Accumulation is fp32.
+ *
+ * Replaces: void sparse_attention_fwd_fp16(const SparseAttentionParams&, cudaStream_t) and
+ *           void sparse_attention_fwd_bf16(const SparseAttentionParams&, cudaStream_t),
+ *           csrc/sparse_attention.h:45-54, defined csrc/sparse_attention.cu:574-601; the
+ *           arguments are the live fields of SparseAttentionParams, csrc/sparse_attention.h:12-38
+ *           (lse == NULL plays the part of is_training == false, csrc/binding.cpp:30).
+ */
+int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *mask_packed,
+                 void *out, float *lse, int B, int H, int N, int D, float scale, int dtype,
+                 void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SMA_H_ */

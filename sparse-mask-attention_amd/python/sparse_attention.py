@@ -1,0 +1,177 @@
+"""Sparse-mask attention: the user-facing Python API, unchanged from the reference.
+
+Mirrors ``python/sparse_attention.py`` of the reference (line numbers below refer to it):
+
+* ``sparse_attention(q, k, v, mask)``       :120-154  autograd-aware entry point
+* ``sparse_attention_func(q, k, v, mask)``  :157-177  inference-only variant (no LSE, no graph)
+* ``pack_mask(mask)``                       :184-201  bool [B,H,N,N] -> int32 [B,H,N,ceil(N/32)]
+* ``SparseAttentionFunction``               :49-113   the autograd.Function behind the first
+* ``sparse_attention_ref``                  :24-42    the plain-PyTorch statement of the operator
+* ``generate_random_sparse_mask``           :204-211
+
+``q, k, v`` are ``[B, H, N, 64]`` fp16 / bf16 tensors on an MI355X (fp32 inputs are computed in
+bf16 and returned as fp32, as in the reference :140-142,151-152); ``mask`` is a bool
+``[B, H, N, N]`` tensor, True = attend.  Query rows that attend to nothing give zeros.
+
+What differs from the reference, on purpose:
+
+* The compute path is the HIP extension ``sparse_attn_cuda`` (same module name) and nothing else.
+  Where the reference silently computes with PyTorch ops when the extension is missing or the
+  tensors live on the CPU (:148-149, :65-74), this module raises ``RuntimeError``: a silent
+  fallback would hide a broken build.  ``sparse_attention_ref`` stays available for callers who
+  want the PyTorch formulation explicitly.
+* ``.backward()`` works.  The reference calls a ``sparse_attn_cuda.backward`` that was never
+  written (:91-94); here the gradient is recomputed on the GPU with PyTorch ops from the saved
+  log-sum-exp, following the reference's own formulas (:97-111).
+"""
+from __future__ import annotations
+
+import math
+import os
+import sys
+
+import torch
+from torch.autograd import Function
+
+_PKG_DIR = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+if _PKG_DIR not in sys.path:
+    sys.path.insert(0, _PKG_DIR)
+
+try:
+    import sparse_attn_cuda  # pybind shim over libsma_hip.so, built in-tree by buildlib.py
+    HAS_CUDA_EXT = True
+    _EXT_ERROR = None
+except ImportError as exc:  # the API stays importable; any compute call reports the cause
+    sparse_attn_cuda = None
+    HAS_CUDA_EXT = False
+    _EXT_ERROR = exc
+
+
+def _require_ext(t: torch.Tensor) -> None:
+    if not HAS_CUDA_EXT:
+        raise RuntimeError(
+            "the HIP extension sparse_attn_cuda is not built or failed to load "
+            f"({_EXT_ERROR}); run `python setup.py build_ext --inplace` in {_PKG_DIR}")
+    if not t.is_cuda:
+        raise RuntimeError("sparse attention runs on the GPU only: move q, k, v and mask to the "
+                           "device (sparse_attention_ref is the PyTorch formulation for any device)")
+
+
+# ----------------------------------------------------------------------------------------------
+# Plain-PyTorch statement of the operator (never called by the functions below)
+# ----------------------------------------------------------------------------------------------
+
+def sparse_attention_ref(q, k, v, mask):
+    """softmax(mask ? q k^T / sqrt(D) : -inf) v with PyTorch ops, in the dtype of the inputs."""
+    scale = 1.0 / math.sqrt(q.shape[-1])
+    logits = (q @ k.transpose(-1, -2)) * scale
+    logits = logits.masked_fill(mask.logical_not(), float("-inf"))
+    probs = torch.nan_to_num(torch.softmax(logits, dim=-1), nan=0.0)   # empty rows -> zeros
+    return probs @ v
+
+
+# ----------------------------------------------------------------------------------------------
+# autograd
+# ----------------------------------------------------------------------------------------------
+
+class SparseAttentionFunction(Function):
+    """forward = fused HIP kernel (saves LSE); backward = recomputation from LSE on the GPU."""
+
+    @staticmethod
+    def forward(ctx, q, k, v, mask_packed, mask_bool, scale, seq_len):
+        _require_ext(q)
+        B, H, N, _ = q.shape
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        out = torch.empty_like(q)
+        lse = torch.empty(B, H, N, device=q.device, dtype=torch.float32)
+        sparse_attn_cuda.forward(q, k, v, mask_packed, out, lse, scale, True)
+        ctx.save_for_backward(q, k, v, out, lse, mask_bool)
+        ctx.scale = scale
+        return out
+
+    @staticmethod
+    def backward(ctx, dout):
+        q, k, v, out, lse, mask_bool = ctx.saved_tensors
+        scale = ctx.scale
+        qf, kf, vf, do = q.float(), k.float(), v.float(), dout.float()
+        # p = exp(s - lse) on kept entries; rows that keep nothing have lse = -inf and p = 0.
+        s = (qf @ kf.transpose(-1, -2)) * scale
+        safe_lse = torch.where(torch.isinf(lse), torch.zeros_like(lse), lse).unsqueeze(-1)
+        p = torch.exp(s - safe_lse).masked_fill(mask_bool.logical_not(), 0.0)
+        dv = p.transpose(-1, -2) @ do
+        dp = do @ vf.transpose(-1, -2)
+        delta = (do * out.float()).sum(dim=-1, keepdim=True)      # = sum_j p_ij dp_ij
+        ds = p * (dp - delta) * scale
+        dq = ds @ kf
+        dk = ds.transpose(-1, -2) @ qf
+        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None
+
+
+# ----------------------------------------------------------------------------------------------
+# public entry points
+# ----------------------------------------------------------------------------------------------
+
+def _check_inputs(q, k, v, mask):
+    assert q.shape == k.shape == v.shape, "q/k/v must have the same shape"
+    assert q.device == k.device == v.device == mask.device, "all tensors must be on the same device"
+    assert mask.dtype == torch.bool, "mask must be a bool tensor"
+
+
+def sparse_attention(q, k, v, mask):
+    """Masked attention with autograd support.
+
+    q, k, v: ``[B, H, N, D]`` (D = 64) bf16 / fp16 / fp32;  mask: bool ``[B, H, N, N]``, True = keep.
+    Returns a tensor of q's shape and original dtype.
+    """
+    _check_inputs(q, k, v, mask)
+    _require_ext(q)
+    B, H, N, D = q.shape
+    scale = 1.0 / math.sqrt(D)
+
+    orig_dtype = q.dtype
+    if orig_dtype == torch.float32:
+        q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+
+    mask_packed = pack_mask(mask)
+    out = SparseAttentionFunction.apply(q, k, v, mask_packed, mask, scale, N)
+
+    if orig_dtype == torch.float32:
+        out = out.float()
+    return out
+
+
+def sparse_attention_func(q, k, v, mask):
+    """Inference-only variant of :func:`sparse_attention`: no autograd graph, no LSE."""
+    _check_inputs(q, k, v, mask)
+    _require_ext(q)
+    D = q.shape[-1]
+    scale = 1.0 / math.sqrt(D)
+
+    orig_dtype = q.dtype
+    if orig_dtype == torch.float32:
+        q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
+
+    with torch.no_grad():
+        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        mask_packed = pack_mask(mask)
+        out = torch.empty_like(q)
+        sparse_attn_cuda.forward(q, k, v, mask_packed, out, None, scale, False)
+
+    if orig_dtype == torch.float32:
+        out = out.float()
+    return out
+
+
+# ----------------------------------------------------------------------------------------------
+# mask helpers
+# ----------------------------------------------------------------------------------------------
+
+def pack_mask(mask: torch.Tensor) -> torch.Tensor:
+    """bool ``[B, H, N, N]`` -> bit-packed int32 ``[B, H, N, ceil(N/32)]`` (bit j of word w = column 32w+j)."""
+    _require_ext(mask)
+    return sparse_attn_cuda.pack_mask(mask)
+
+
+def generate_random_sparse_mask(B, H, N, sparsity=0.75, device="cuda"):
+    """Random mask whose entries are False (masked out) with probability ``sparsity``."""
+    return torch.rand(B, H, N, N, device=device) > sparsity

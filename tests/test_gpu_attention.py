@@ -1,0 +1,227 @@
+"""GPU parity of sma_attn_fwd (through the C ABI) against the fp32 oracle.
+
+Tolerances: fp16  allclose(atol=1e-2, rtol=1e-2) and the reference's own bar max|diff| < 1e-2
+(run.py:357,371-373); bf16 allclose(atol=1e-2, rtol=2e-2).  Exact equality where the mathematics
+gives it (one-hot rows, empty rows).
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import _capi
+import harness
+from oracle import sma_oracle as O
+from oracle import sma_oracle_c as OC
+
+pytestmark = pytest.mark.gpu
+
+TOL = {torch.float16: dict(atol=1e-2, rtol=1e-2), torch.bfloat16: dict(atol=1e-2, rtol=2e-2)}
+
+
+def _run(q, k, v, mask, dev, scale=None, want_lse=False, packed=None):
+    qd, kd, vd = (t.to(dev) for t in (q, k, v))
+    if packed is None:
+        packed = torch.from_numpy(O.pack_mask_ref(mask)).to(dev)     # oracle-packed: isolates the kernel
+    res = _capi.attn_fwd(qd, kd, vd, packed, scale=scale, want_lse=want_lse)
+    torch.cuda.synchronize()
+    return res
+
+
+def _rand_qkv(B, H, N, dtype, seed, std=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return [(torch.randn(B, H, N, 64, generator=g) * std).to(dtype) for _ in range(3)], g
+
+
+def _assert_close(out, ref, dtype, what=""):
+    out = out.float().cpu()
+    assert not torch.isnan(out).any(), f"{what}: NaN in output"
+    diff = (out - ref).abs()
+    tol = TOL[dtype]
+    bad = diff > tol["atol"] + tol["rtol"] * ref.abs()
+    assert not bad.any(), f"{what}: {int(bad.sum())} elements out of tolerance, max abs diff {diff.max():.4e}"
+    return diff.max().item()
+
+
+@pytest.mark.parametrize("N", [64, 128, 256, 512])
+def test_reference_correctness_run_fp16(dev, N):
+    """The reference's own acceptance run: B=2, H=4, D=64, 75 % sparse, max abs diff < 1e-2."""
+    (q, k, v), g = _rand_qkv(2, 4, N, torch.float16, 42)
+    mask = torch.rand(2, 4, N, N, generator=g) > 0.75
+    out = _run(q, k, v, mask, dev)
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    assert _assert_close(out, ref, torch.float16, f"N={N}") < 1e-2
+
+
+def test_fully_masked_row_gives_zeros_not_nan(dev):
+    """The reference's N=8 case (run.py:387-396), strengthened from 'no NaN' to 'exact zeros'."""
+    (q, k, v), _ = _rand_qkv(1, 1, 8, torch.float16, 1)
+    mask = torch.ones(1, 1, 8, 8, dtype=torch.bool)
+    mask[:, :, 0, :] = False
+    out, lse = _run(q, k, v, mask, dev, want_lse=True)
+    assert not torch.isnan(out).any()
+    assert torch.equal(out[0, 0, 0].cpu(), torch.zeros(64, dtype=torch.float16))
+    assert lse[0, 0, 0].item() == -math.inf
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    _assert_close(out, ref, torch.float16)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("N", [1, 2, 31, 33, 63, 65, 127, 129, 200, 513, 1000])
+def test_ragged_lengths(dev, dtype, N):
+    (q, k, v), g = _rand_qkv(1, 3, N, dtype, 7 + N)
+    mask = torch.rand(1, 3, N, N, generator=g) > 0.7
+    if N > 4:
+        mask[0, 1, 3, :] = False
+    out, lse = _run(q, k, v, mask, dev, want_lse=True)
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    _assert_close(out, ref, dtype, f"N={N}")
+    lse_ref = O.lse_ref(q, k, mask)
+    fin = torch.isfinite(lse_ref)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    assert torch.allclose(lse.cpu()[fin], lse_ref[fin], atol=2e-3, rtol=1e-3)
+    assert (lse.cpu()[~fin] == -math.inf).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_one_hot_rows_are_exact(dev, dtype):
+    N = 192
+    (q, k, v), g = _rand_qkv(2, 2, N, dtype, 3)
+    perm = torch.stack([torch.randperm(N, generator=g) for _ in range(4)]).view(2, 2, N)
+    mask = torch.zeros(2, 2, N, N, dtype=torch.bool)
+    mask.scatter_(3, perm.unsqueeze(-1), True)
+    out = _run(q, k, v, mask, dev).cpu()
+    expect = torch.gather(v, 2, perm.unsqueeze(-1).expand(-1, -1, -1, 64))
+    assert torch.equal(out, expect)          # p == 1 exactly: the output is the selected value row
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_all_true_and_all_false_masks(dev, dtype):
+    N = 160
+    (q, k, v), _ = _rand_qkv(1, 2, N, dtype, 4)
+    mask = torch.ones(1, 2, N, N, dtype=torch.bool)
+    ref = torch.nn.functional.scaled_dot_product_attention(q.float(), k.float(), v.float())
+    _assert_close(_run(q, k, v, mask, dev), ref, dtype, "all true")
+    out, lse = _run(q, k, v, ~mask, dev, want_lse=True)
+    assert (out == 0).all() and (lse == -math.inf).all()
+
+
+def test_large_masked_scores_do_not_disturb_kept_ones(dev):
+    """Dropped keys with huge scores must not enter the running maximum."""
+    N = 128
+    (q, k, v), g = _rand_qkv(1, 2, N, torch.float16, 5)
+    mask = torch.rand(1, 2, N, N, generator=g) > 0.5
+    mask[..., 0::2] = False                      # drop the even keys ...
+    k[:, :, 0::2, :] = q[:, :, 0::2, :] * 30.0   # ... and give them enormous scores for many queries
+    mask[..., 1] = True
+    out = _run(q, k, v, mask, dev)
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    _assert_close(out, ref, torch.float16)
+
+
+def test_large_kept_scores_are_stable(dev):
+    N = 96
+    (q, k, v), g = _rand_qkv(1, 1, N, torch.float16, 6)
+    q *= 12.0                                    # logits of magnitude ~100
+    mask = torch.rand(1, 1, N, N, generator=g) > 0.3
+    out = _run(q, k, v, mask, dev)
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    _assert_close(out, ref, torch.float16)
+
+
+@pytest.mark.parametrize("scale", [0.125, 1.0, 0.01, -0.125, 0.0])
+def test_scale_argument(dev, scale):
+    N = 100
+    (q, k, v), g = _rand_qkv(1, 2, N, torch.float16, 8)
+    mask = torch.rand(1, 2, N, N, generator=g) > 0.6
+    out, lse = _run(q, k, v, mask, dev, scale=scale, want_lse=True)
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask, scale=scale)
+    _assert_close(out, ref, torch.float16, f"scale={scale}")
+    lse_ref = O.lse_ref(q, k, mask, scale=scale)
+    fin = torch.isfinite(lse_ref)
+    assert torch.allclose(lse.cpu()[fin], lse_ref[fin], atol=2e-3, rtol=1e-3)
+
+
+def test_pad_bits_of_the_packed_mask_are_ignored(dev):
+    N = 100                                      # 4 words per row, 28 pad bits in the last one
+    (q, k, v), g = _rand_qkv(1, 2, N, torch.float16, 9)
+    mask = torch.rand(1, 2, N, N, generator=g) > 0.6
+    packed = O.pack_mask_ref(mask).view(np.uint32).copy()
+    dirty = packed.copy()
+    dirty[..., -1] |= np.uint32(0xFFFFFFF0)
+    a = _run(q, k, v, mask, dev, packed=torch.from_numpy(packed.view(np.int32)).to(dev))
+    b = _run(q, k, v, mask, dev, packed=torch.from_numpy(dirty.view(np.int32)).to(dev))
+    assert torch.equal(a, b)
+
+
+def test_empty_tiles_and_rows_are_skipped_correctly(dev):
+    """64x64 block-structured mask with empty block rows, empty tiles and full tiles."""
+    N = 448                                      # 7 blocks: last query tile of 128 is half empty
+    (q, k, v), g = _rand_qkv(2, 2, N, torch.float16, 10)
+    blocks = torch.rand(2, 2, 7, 7, generator=g) > 0.7
+    blocks[:, :, 2, :] = False                   # a whole block row keeps nothing
+    mask = blocks.repeat_interleave(64, 2).repeat_interleave(64, 3)
+    out = _run(q, k, v, mask, dev)
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    _assert_close(out, ref, torch.float16)
+    assert (out[:, :, 128:192] == 0).all()
+
+
+def test_rows_are_independent_and_deterministic(dev):
+    N = 256
+    (q, k, v), g = _rand_qkv(1, 2, N, torch.float16, 11)
+    mask = torch.rand(1, 2, N, N, generator=g) > 0.75
+    a = _run(q, k, v, mask, dev)
+    b = _run(q, k, v, mask, dev)
+    assert torch.equal(a, b)
+    mask2 = mask.clone()
+    mask2[:, :, 77, :] = ~mask2[:, :, 77, :]
+    c = _run(q, k, v, mask2, dev)
+    keep = torch.arange(N) != 77
+    assert torch.equal(a[:, :, keep], c[:, :, keep])
+
+
+def test_c_oracle_agrees_on_a_small_case(dev):
+    N = 80
+    (q, k, v), g = _rand_qkv(1, 2, N, torch.float16, 12)
+    mask = torch.rand(1, 2, N, N, generator=g) > 0.75
+    out, lse = _run(q, k, v, mask, dev, want_lse=True)
+    ref, lse_ref = OC.attn_fwd(q.float().numpy(), k.float().numpy(), v.float().numpy(), mask.numpy(), 0.125)
+    _assert_close(out, torch.from_numpy(ref), torch.float16)
+    assert np.allclose(lse.cpu().numpy(), lse_ref, atol=2e-3)
+
+
+def _head_subset(w, n, seed):
+    idx = torch.randperm(w.B * w.H, generator=torch.Generator().manual_seed(seed))[:n].tolist()
+    idx = sorted(set(idx) | {0, w.B * w.H - 1})
+    return [(i // w.H, i % w.H) for i in idx]
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
+def test_benchmark_workloads(dev, name):
+    """The five benchmark configurations at full size, packed by the HIP packer.
+
+    The oracle is evaluated on every head for C1/C2 and on a seeded subset of heads (first and last
+    included) for the larger ones; the whole output is additionally checked through a property that
+    needs no oracle: with V = 1 every row that keeps a key must come out as exactly 1."""
+    w = harness.WORKLOADS[name]
+    q, k, v, mask = harness.make_inputs(w, seed=42)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    packed = _capi.pack_mask(md)
+    out = _capi.attn_fwd(qd, kd, vd, packed)
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()
+    heads = [(b, h) for b in range(w.B) for h in range(w.H)] if name in ("C1", "C2") else _head_subset(w, 12, 1)
+    outc = out.cpu()
+    worst = 0.0
+    for b, h in heads:
+        sl = (slice(b, b + 1), slice(h, h + 1))
+        ref = O.sparse_attention_ref(q[sl].float(), k[sl].float(), v[sl].float(), mask[sl])
+        worst = max(worst, _assert_close(outc[sl], ref, w.dtype, f"{name} head {(b, h)}"))
+    print(f"{name}: max abs diff over {len(heads)} heads = {worst:.3e}")
+    ones = torch.ones_like(vd)
+    out1 = _capi.attn_fwd(qd, kd, ones, packed)
+    torch.cuda.synchronize()
+    nonempty = md.any(dim=-1, keepdim=True).expand(-1, -1, -1, 64)
+    assert torch.equal(out1.float(), nonempty.float())

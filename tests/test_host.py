@@ -1,0 +1,132 @@
+"""CPU-only checks of the host side: the C ABI loads and exports what include/sma.h declares,
+argument validation answers before anything touches a GPU, the Python API keeps the reference's
+surface and refuses to compute anywhere but on the device, and the workloads have the documented
+sizes."""
+import ctypes
+import os
+import re
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import _capi
+import harness
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol(capi):
+    header = open(os.path.join(ROOT, "include", "sma.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(sma_[a-z_0-9]+)\s*\(", header))
+    assert {"sma_version", "sma_strerror", "sma_pack_mask", "sma_attn_fwd"} <= declared
+    for name in declared:
+        assert hasattr(capi, name), f"{name} is declared in sma.h but not exported"
+    assert capi.sma_version() >= 100
+    assert capi.sma_strerror(0) == b"ok"
+    for code in range(-7, 0):
+        assert capi.sma_strerror(code) not in (b"ok", b"unknown error code")
+    assert capi.sma_strerror(-99) == b"unknown error code"
+
+
+def test_argument_validation_needs_no_gpu(capi):
+    p = ctypes.c_void_p(0x1000)            # never dereferenced: every call below fails or is a no-op first
+    f = capi.sma_attn_fwd
+    ok_args = dict(B=1, H=1, N=64, D=64, scale=0.125, dtype=_capi.SMA_DTYPE_F16)
+
+    def call(q=p, k=p, v=p, mp=p, out=p, lse=None, **kw):
+        a = dict(ok_args, **kw)
+        return f(q, k, v, mp, out, lse, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
+
+    assert call(D=32) == _capi.SMA_ERR_HEAD_DIM
+    assert call(D=128) == _capi.SMA_ERR_HEAD_DIM
+    assert call(dtype=2) == _capi.SMA_ERR_DTYPE
+    assert call(B=-1) == _capi.SMA_ERR_BAD_SHAPE
+    assert call(scale=float("nan")) == _capi.SMA_ERR_SCALE
+    assert call(scale=float("inf")) == _capi.SMA_ERR_SCALE
+    assert call(q=None) == _capi.SMA_ERR_NULL_POINTER
+    assert call(out=None) == _capi.SMA_ERR_NULL_POINTER
+    assert call(q=ctypes.c_void_p(0x1002)) == _capi.SMA_ERR_ALIGNMENT
+    assert call(B=0) == _capi.SMA_OK and call(N=0) == _capi.SMA_OK          # empty problem: nothing to do
+    assert call(B=1 << 20, H=1 << 12, N=64) == _capi.SMA_ERR_BAD_SHAPE      # index range
+
+    g = capi.sma_pack_mask
+    assert g(None, p, 1, 1, 8, None) == _capi.SMA_ERR_NULL_POINTER
+    assert g(p, None, 1, 1, 8, None) == _capi.SMA_ERR_NULL_POINTER
+    assert g(p, p, 1, -2, 8, None) == _capi.SMA_ERR_BAD_SHAPE
+    assert g(p, p, 0, 4, 8, None) == _capi.SMA_OK
+    assert g(p, ctypes.c_void_p(0x1001), 1, 1, 8, None) == _capi.SMA_ERR_ALIGNMENT
+
+
+def test_python_api_surface_and_loud_failure_off_gpu():
+    import python as pkg
+    assert set(pkg.__all__) == {"sparse_attention", "sparse_attention_func"}
+    sa = sys.modules["python.sparse_attention"]
+    for name in ("sparse_attention", "sparse_attention_func", "pack_mask", "sparse_attention_ref",
+                 "SparseAttentionFunction", "generate_random_sparse_mask", "HAS_CUDA_EXT"):
+        assert hasattr(sa, name), name
+    assert sa.HAS_CUDA_EXT, f"extension did not import: {sa._EXT_ERROR}"
+    import sparse_attn_cuda
+    assert {"forward", "pack_mask"} <= set(dir(sparse_attn_cuda))
+    q = torch.randn(1, 1, 8, 64)
+    m = torch.ones(1, 1, 8, 8, dtype=torch.bool)
+    for fn in (sa.sparse_attention, sa.sparse_attention_func):
+        with pytest.raises(RuntimeError, match="GPU only"):
+            fn(q, q, q, m)
+    with pytest.raises(RuntimeError, match="GPU only"):
+        sa.pack_mask(m)
+    with pytest.raises(AssertionError):
+        sa.sparse_attention(q, q, q, m.to(torch.uint8))
+    with pytest.raises(AssertionError):
+        sa.sparse_attention(q, q[:, :, :4], q, m)
+    # the binding itself rejects host tensors with the reference's RuntimeError convention
+    with pytest.raises(RuntimeError):
+        sparse_attn_cuda.pack_mask(m)
+    with pytest.raises(RuntimeError):
+        sparse_attn_cuda.forward(q.half(), q.half(), q.half(), torch.zeros(1, 1, 8, 1, dtype=torch.int32),
+                                 q.half(), None, 0.125, False)
+
+
+def test_reference_formulation_kept_in_the_api_matches_the_oracle():
+    from oracle import sma_oracle as O
+    sa = sys.modules.get("python.sparse_attention") or __import__("python.sparse_attention")
+    sa = sys.modules["python.sparse_attention"]
+    q, k, v, mask = harness.make_inputs("C1", seed=1)
+    mask[0, 0, 3, :] = False
+    a = sa.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    b = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    assert torch.equal(a, b)
+
+
+def test_workload_shapes_and_algorithmic_sizes():
+    W = harness.WORKLOADS
+    assert (W["C2"].B, W["C2"].H, W["C2"].N, W["C2"].D) == (16, 12, 512, 64)
+    assert W["C2"].dense_flops == 12884901888
+    assert W["C2"].attn_bytes == 56623104 and W["C2"].pack_bytes == 56623104
+    assert W["C3"].attn_bytes == 125829120 and W["C3"].pack_bytes == 226492416
+    assert W["C4"].attn_bytes == 81920000 and W["C4"].pack_bytes == 144384000
+    assert W["C5"].attn_bytes == 142606336 and W["C5"].pack_bytes == 75497472
+    q, k, v, m = harness.make_inputs("C1", seed=42)
+    assert q.shape == (1, 2, 128, 64) and q.dtype == torch.float16 and m.dtype == torch.bool
+    assert 0.2 < m.float().mean() < 0.3
+    q2, _, _, m2 = harness.make_inputs("C1", seed=42)
+    assert torch.equal(q, q2) and torch.equal(m, m2)                       # deterministic
+
+
+def test_structured_masks():
+    small = harness.Workload("blk", 1, 2, 256, 64, torch.float16, "block64", 0.25)
+    m = harness.make_mask(small, torch.Generator().manual_seed(0))
+    t = m.reshape(1, 2, 4, 64, 4, 64)
+    per_block = t.float().mean(dim=(3, 5))
+    assert ((per_block == 0) | (per_block == 1)).all()
+    assert (torch.diagonal(per_block, dim1=2, dim2=3) == 1).all()
+    rag = harness.Workload("rag", 1, 1, 100, 64, torch.bfloat16, "random_diag", 0.1, 0.5)
+    m = harness.make_mask(rag, torch.Generator().manual_seed(0))
+    assert torch.diagonal(m[0, 0]).all() and m.float().mean() < 0.2
+    cau = harness.Workload("cau", 1, 1, 64, 64, torch.float16, "causal_random", 0.5)
+    m = harness.make_mask(cau, torch.Generator().manual_seed(0))
+    assert not torch.triu(m[0, 0], diagonal=1).any() and torch.diagonal(m[0, 0]).all()
+    tf, pct = harness.compute_mfu(1.0, 16, 12, 512, 64, 2516.6)
+    assert tf == pytest.approx(12.884901888) and pct == pytest.approx(100 * 12.884901888 / 2516.6)

@@ -1,0 +1,186 @@
+"""Pins of the CPU oracle (no GPU): library routines, known answers, closed forms, brute force.
+
+The reference ships no golden vectors for this path (its only checks are tolerance runs against
+its own PyTorch formulation on CUDA-seeded inputs, run.py:355-376 and :387-396), so the oracle is
+pinned by what the format and the mathematics fix.  Each test is chosen so that a plausible slip
+(MSB-first bits, wrong word order, non-zero pad bits, a transposed operand, a missing scale, a
+wrong empty-row convention) fails it.
+"""
+import math
+
+import numpy as np
+import pytest
+import scipy.special
+import torch
+
+from oracle import sma_oracle as O
+from oracle import sma_oracle_c as OC
+
+
+# ---------------------------------------------------------------- pack format
+
+def test_pack_single_bit_known_answers():
+    N = 70
+    for c in (0, 1, 31, 32, 33, 63, 64, 69):
+        m = np.zeros((1, 1, N, N), dtype=bool)
+        m[0, 0, 5, c] = True
+        p = O.pack_mask_ref(m).view(np.uint32)
+        assert p.shape == (1, 1, N, 3)
+        expect = np.zeros((N, 3), dtype=np.uint32)
+        expect[5, c // 32] = np.uint32(1) << np.uint32(c % 32)
+        assert np.array_equal(p[0, 0], expect), c
+    # column 31 sets the sign bit of the int32 word, as `int32 << 31` does in the reference's
+    # CPU fallback (python/sparse_attention.py:195-200)
+    m = np.zeros((1, 1, 32, 32), dtype=bool)
+    m[0, 0, 0, 31] = True
+    assert O.pack_mask_ref(m)[0, 0, 0, 0] == -2**31
+
+
+def test_pack_all_true_tail_words():
+    p = O.pack_mask_ref(np.ones((1, 1, 8, 8), dtype=bool)).view(np.uint32)
+    assert p.shape == (1, 1, 8, 1) and (p == 0xFF).all()
+    p = O.pack_mask_ref(np.ones((1, 2, 1000, 1000), dtype=bool)).view(np.uint32)
+    assert p.shape == (1, 2, 1000, 32)
+    assert (p[..., :31] == 0xFFFFFFFF).all() and (p[..., 31] == 0xFF).all()   # 1000 = 31*32 + 8
+    assert O.pack_mask_ref(np.ones((1, 1, 33, 33), dtype=bool)).dtype == np.int32
+
+
+@pytest.mark.parametrize("N", [1, 8, 31, 32, 33, 64, 100])
+def test_pack_three_statements_agree(N):
+    rng = np.random.default_rng(N)
+    m = rng.random((2, 3, N, N)) > 0.6
+    a = O.pack_mask_ref(m)
+    assert np.array_equal(a, O.pack_mask_loops(m))       # literal bit loop (Python)
+    assert np.array_equal(a, OC.pack_mask(m))            # literal bit loop (C)
+
+
+@pytest.mark.parametrize("N", [8, 33, 64, 257, 1000])
+def test_pack_invariants(N):
+    rng = np.random.default_rng(7 * N)
+    m = rng.random((1, 2, N, N)) > 0.75
+    p = O.pack_mask_ref(m)
+    assert np.array_equal(O.unpack_mask_ref(p, N), m)                       # round trip
+    bits = np.unpackbits(p.view(np.uint8), bitorder="little").sum()
+    assert bits == m.sum()                                                  # popcount, pad bits 0
+    tail = N % 32
+    if tail:
+        assert (p.view(np.uint32)[..., -1] >> np.uint32(tail) == 0).all()
+
+
+def test_pack_accepts_torch_and_matches_reference_cpu_formula():
+    # the reference's CPU fallback builds words with `|= mask[..., col].int() << bit`
+    g = torch.Generator().manual_seed(3)
+    m = torch.rand(1, 2, 40, 40, generator=g) > 0.5
+    nw = 2
+    expect = torch.zeros(1, 2, 40, nw, dtype=torch.int32)
+    for col in range(40):
+        expect[..., col // 32] |= m[..., col].int() << (col % 32)
+    assert np.array_equal(O.pack_mask_ref(m), expect.numpy())
+
+
+# ---------------------------------------------------------------- attention
+
+def _rand(B, H, N, D, seed, dtype=torch.float32):
+    g = torch.Generator().manual_seed(seed)
+    return [torch.randn(B, H, N, D, generator=g).to(dtype).float() for _ in range(3)]
+
+
+def test_all_true_mask_is_dense_attention():
+    q, k, v = _rand(2, 3, 50, 64, 0)
+    mask = torch.ones(2, 3, 50, 50, dtype=torch.bool)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v)
+    assert torch.allclose(O.sparse_attention_ref(q, k, v, mask), ref, atol=1e-5, rtol=1e-5)
+
+
+def test_bool_mask_matches_sdpa_on_nonempty_rows():
+    q, k, v = _rand(1, 2, 40, 64, 1)
+    g = torch.Generator().manual_seed(11)
+    mask = (torch.rand(1, 2, 40, 40, generator=g) > 0.75) | torch.eye(40, dtype=torch.bool)
+    ref = torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask)   # True = keep
+    assert torch.allclose(O.sparse_attention_ref(q, k, v, mask), ref, atol=1e-5, rtol=1e-5)
+
+
+def test_one_hot_rows_return_the_selected_value_row():
+    q, k, v = _rand(1, 1, 16, 64, 2)
+    perm = torch.randperm(16, generator=torch.Generator().manual_seed(5))
+    mask = torch.zeros(1, 1, 16, 16, dtype=torch.bool)
+    mask[0, 0, torch.arange(16), perm] = True
+    out = O.sparse_attention_ref(q, k, v, mask)
+    assert torch.equal(out[0, 0], v[0, 0, perm])       # a transposed mask would give v[inverse perm]
+
+
+def test_empty_rows_give_zeros_and_minus_inf_lse():
+    q, k, v = _rand(1, 1, 8, 64, 3)
+    mask = torch.ones(1, 1, 8, 8, dtype=torch.bool)
+    mask[0, 0, 0, :] = False                            # the reference's own case, run.py:387-396
+    out = O.sparse_attention_ref(q, k, v, mask)
+    assert not torch.isnan(out).any()
+    assert torch.equal(out[0, 0, 0], torch.zeros(64))
+    lse = O.lse_ref(q, k, mask)
+    assert lse[0, 0, 0] == -math.inf and torch.isfinite(lse[0, 0, 1:]).all()
+
+
+def test_zero_queries_give_mean_of_kept_values():
+    _, k, v = _rand(1, 2, 30, 64, 4)
+    q = torch.zeros(1, 2, 30, 64)
+    g = torch.Generator().manual_seed(9)
+    mask = (torch.rand(1, 2, 30, 30, generator=g) > 0.5) | torch.eye(30, dtype=torch.bool)
+    out = O.sparse_attention_ref(q, k, v, mask)
+    w = mask.float() / mask.float().sum(-1, keepdim=True)
+    assert torch.allclose(out, w @ v, atol=1e-6, rtol=1e-5)
+
+
+def test_scale_is_one_over_sqrt_d_and_enters_the_scores():
+    # two keys, scores differ by a known amount: softmax weights have a closed form
+    D = 64
+    q = torch.zeros(1, 1, 2, D); q[..., 0] = 8.0
+    k = torch.zeros(1, 1, 2, D); k[0, 0, 1, 0] = 1.0      # scores (0, 8) -> scaled (0, 1)
+    v = torch.zeros(1, 1, 2, D); v[0, 0, 0, 0] = 1.0; v[0, 0, 1, 1] = 1.0
+    mask = torch.ones(1, 1, 2, 2, dtype=torch.bool)
+    out = O.sparse_attention_ref(q, k, v, mask)
+    p1 = math.e / (1.0 + math.e)
+    assert out[0, 0, 0, 1].item() == pytest.approx(p1, rel=1e-6)
+    assert out[0, 0, 0, 0].item() == pytest.approx(1.0 - p1, rel=1e-6)
+    assert O.lse_ref(q, k, mask)[0, 0, 0].item() == pytest.approx(math.log(1.0 + math.e), rel=1e-6)
+
+
+def test_key_permutation_invariance_and_row_independence():
+    q, k, v = _rand(1, 2, 24, 64, 5)
+    g = torch.Generator().manual_seed(13)
+    mask = (torch.rand(1, 2, 24, 24, generator=g) > 0.6) | torch.eye(24, dtype=torch.bool)
+    out = O.sparse_attention_ref(q, k, v, mask)
+    perm = torch.randperm(24, generator=g)
+    out_p = O.sparse_attention_ref(q, k[:, :, perm], v[:, :, perm], mask[:, :, :, perm])
+    assert torch.allclose(out, out_p, atol=1e-6, rtol=1e-5)
+    mask2 = mask.clone()
+    mask2[:, :, 7, :] = ~mask2[:, :, 7, :]
+    out2 = O.sparse_attention_ref(q, k, v, mask2)
+    keep = torch.arange(24) != 7
+    assert torch.equal(out[:, :, keep], out2[:, :, keep])
+
+
+@pytest.mark.parametrize("N", [8, 33, 70])
+def test_torch_numpy_and_c_statements_agree(N):
+    q, k, v = _rand(1, 2, N, 64, 6 + N, dtype=torch.float16)
+    g = torch.Generator().manual_seed(17)
+    mask = torch.rand(1, 2, N, N, generator=g) > 0.75
+    mask[0, 0, 1, :] = False
+    scale = 1.0 / 8.0
+    a = O.sparse_attention_ref(q, k, v, mask).numpy()
+    b, lse_b = O.attention_f64_loops(q.numpy(), k.numpy(), v.numpy(), mask)
+    c, lse_c = OC.attn_fwd(q.numpy(), k.numpy(), v.numpy(), mask.numpy(), scale)
+    assert np.allclose(a, b, atol=2e-6, rtol=1e-5)
+    assert np.allclose(c, b, atol=2e-6, rtol=1e-5)
+    lse_a = O.lse_ref(q, k, mask).numpy()
+    assert np.allclose(lse_a, lse_b, atol=1e-5, equal_nan=False)
+    assert np.allclose(lse_c, lse_b, atol=1e-5)
+    assert lse_a[0, 0, 1] == -np.inf and lse_c[0, 0, 1] == -np.inf
+
+
+def test_lse_matches_scipy_logsumexp():
+    q, k, _ = _rand(1, 1, 12, 64, 8)
+    g = torch.Generator().manual_seed(19)
+    mask = (torch.rand(1, 1, 12, 12, generator=g) > 0.5) | torch.eye(12, dtype=torch.bool)
+    s = (q[0, 0] @ k[0, 0].T).numpy() / 8.0
+    expect = np.array([scipy.special.logsumexp(s[i][mask[0, 0, i].numpy()]) for i in range(12)])
+    assert np.allclose(O.lse_ref(q, k, mask)[0, 0].numpy(), expect, atol=1e-5)
