@@ -231,9 +231,8 @@ __global__ __launch_bounds__(NTHREADS) void attn_fwd_kernel(const AttnArgs a)
                 for (int g = 0; g < 4; ++g)
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
-                        const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)wsh, 8 * g + j, 1);
-                        const uint32_t sb = __builtin_bit_cast(uint32_t, sacc[blk][4 * g + j]);
-                        const float sv = __builtin_bit_cast(float, (sb & keep) | (NEG_INF_BITS & ~keep));
+                        const bool keep = ((wsh >> (8 * g + j)) & 1u) != 0u;
+                        const float sv = keep ? sacc[blk][4 * g + j] : -__builtin_inff();
                         sacc[blk][4 * g + j] = sv;
                         mx = __builtin_fmaxf(mx, sv);
                     }
