@@ -70,17 +70,23 @@ int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *ma
     a.N = N;
     a.nw = (N + 31) / 32;
     a.qtiles = (int)qtiles;
-    // exp(scale*s - max) is evaluated as exp2(c*s' - c*max') with c = |scale|*log2(e) > 0 and
-    // s' = s for scale > 0, s' = -s (q negated on load, exact) for scale < 0.  scale == 0 uses a
-    // denormal-free tiny c: kept scores all map to exp2(~0) = 1, dropped ones stay at -inf.
+    // exp(scale*s) = exp2(post_mul * (q_scale*q).k) with q_scale*post_mul = scale*log2(e), post_mul a
+    // power of two >= 1 chosen so that |q_scale| <= 1: scaling q cannot overflow its 16-bit format.
     const float LOG2E = 1.4426950408889634f;
-    float c = fabsf(scale) * LOG2E;
-    if (!(c > 0.0f)) c = 1e-30f;
-    a.c = c;
-    a.scale_abs = fabsf(scale);
-    a.qsign = (scale < 0.0f) ? 0x80008000u : 0u;
-    const int tail = N & 31;
-    a.tail_mask = tail ? ((1u << tail) - 1u) : 0xffffffffu;
+    const float c = fabsf(scale) * LOG2E;
+    float post_mul = 1.0f;
+    if (c > 1.0f) {
+        int e = 0;
+        (void)frexpf(c, &e);                    // c = f * 2^e, f in [0.5, 1)
+        post_mul = ldexpf(1.0f, e);
+    }
+    a.q_scale = (scale < 0.0f ? -c : c) / post_mul;
+    a.post_mul = post_mul;
+    const int T = (N + 63) / 64;
+    const int rem = N - 64 * (T - 1);           // keys in the last tile, 1..64
+    const int v0 = rem < 32 ? rem : 32, v1 = rem > 32 ? rem - 32 : 0;
+    a.last_mask0 = v0 >= 32 ? 0xffffffffu : ((1u << v0) - 1u);
+    a.last_mask1 = v1 >= 32 ? 0xffffffffu : ((1u << v1) - 1u);
 
     const hipError_t e = sma::launch_attn_fwd(a, dtype == SMA_DTYPE_BF16, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;

@@ -15,10 +15,12 @@ struct AttnArgs {
     float *lse;                     // [BH, N] or nullptr
     int BH, N, nw;
     int qtiles;                     // ceil(N / 128): query tiles (work-groups) per (b,h)
-    float c;                        // |scale| * log2(e), > 0
-    float scale_abs;                // |scale|
-    uint32_t qsign;                 // 0x80008000 when scale < 0 (q is negated on load), else 0
-    uint32_t tail_mask;             // valid-bit mask of the last word of a mask row
+    // exp(scale * s) is evaluated as exp2(post_mul * (q_scale * q) . k): q is multiplied by
+    // q_scale (sign of scale included, |q_scale| <= 1) when it is loaded, post_mul is a power of
+    // two that is 1 unless |scale| * log2(e) > 1.
+    float q_scale;
+    float post_mul;
+    uint32_t last_mask0, last_mask1;   // valid-bit masks of the two mask words of the last key tile
 };
 
 hipError_t launch_attn_fwd(const AttnArgs &a, bool bf16, hipStream_t stream);
