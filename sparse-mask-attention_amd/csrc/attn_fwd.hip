@@ -36,6 +36,8 @@
 //   skipping    = the work-group keeps a per-tile flag "some mask bit of my 128 rows is set",
 //                 computed two tiles ahead: tiles without it are never loaded or computed; and a
 //                 wavefront whose own 32x64 block of bits is empty skips its work for that tile.
+#include <type_traits>
+
 #include "sma_internal.h"
 
 namespace sma {
@@ -62,10 +64,10 @@ constexpr float WINDOW_LOG2 = 8.0f;
 
 // LDS map (bytes)
 constexpr int STAGE_BYTES = 2 * TILE_BYTES;                 // K then V
-constexpr int OFF_MASK = NSTAGE * STAGE_BYTES;              // 4 slots x 4 waves x 64 words
-constexpr int OFF_LUT = OFF_MASK + 4 * 1024;                // 16 x 16 B
-constexpr int OFF_LIVE = OFF_LUT + 256;                     // 4 words
-constexpr int LDS_BYTES = OFF_LIVE + 16;
+constexpr int OFF_MASK = NSTAGE * STAGE_BYTES;              // 3 slots x 4 waves x 64 words
+constexpr int OFF_LUT = OFF_MASK + 3 * 1024;                // 16 x 16 B
+constexpr int OFF_LIVE = OFF_LUT + 256;                     // 3 slots x 4 waves, one word each
+constexpr int LDS_BYTES = OFF_LIVE + 48;
 
 template <bool BF16> struct Elem;
 
@@ -190,32 +192,34 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     const uint16_t *vb = a.v + (size_t)bh * N * HD;
     const uint32_t *mb = a.mask_packed + (size_t)bh * N * nw;
 
-    // ---- small LDS tables ----
-    // entry n (16 B) of the mask table holds four floats, float j = (bit j of n) ? 0 : -inf
-    if (tid < 64)
-        reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
-    uint32_t *s_live = reinterpret_cast<uint32_t *>(smem + OFF_LIVE);
-    if (tid < 4) s_live[tid] = 0u;
-
-    // ---- mask words: wave-private async copies, slot = tile & 3, lane i -> (row i/2, word i%2) ----
+    // ---- mask words: wave-private async copies, slot = tile % 3, lane i -> (row i/2, word i%2) ----
     const int mrow = qt * BM + wave * 32 + (lane >> 1);
     const uint32_t m_voff = (uint32_t)(((size_t)(mrow < N ? mrow : N - 1) * nw + (lane & 1)) * 4);
-    auto issue_mask = [&](int x) {
+    auto issue_mask = [&](int x, int slot) {
         const int xt = x < T ? x : T - 1;
-        const uint32_t dst = lds0 + OFF_MASK + (x & 3) * 1024 + wave * 256;
+        const uint32_t dst = lds0 + OFF_MASK + slot * 1024 + wave * 256;
         uint32_t voff = m_voff;
         if (2 * xt + 1 >= nw) voff -= (lane & 1) * 4;          // odd word count: re-read the last word
         async_copy_b32(dst, mb + 2 * xt, voff);
     };
     const uint32_t maddr = lds0 + OFF_MASK + wave * 256 + l32 * 8;
-    auto mask_words = [&](int x) -> u32x2 {
-        u32x2 w = lds_read_b64(maddr + (x & 3) * 1024);
-        if (x == T - 1) { w.x &= a.last_mask0; w.y &= a.last_mask1; }
+    auto mask_words = [&](int x, int slot) -> u32x2 {
+        u32x2 w = lds_read_b64(maddr + slot * 1024);
+        const bool last = (x == T - 1);
+        w.x &= last ? a.last_mask0 : 0xffffffffu;
+        w.y &= last ? a.last_mask1 : 0xffffffffu;
         return w;
     };
-    auto mark_live = [&](int x) {
-        const u32x2 w = mask_words(x);
-        if (__builtin_amdgcn_ballot_w64((w.x | w.y) != 0u) != 0ull && lane == 0) atomicOr(&s_live[x & 3], 1u);
+    // flag "some mask bit of tile x is set in this wave's 32 rows", one word per (slot, wave)
+    uint32_t *s_live = reinterpret_cast<uint32_t *>(smem + OFF_LIVE);
+    auto mark_live = [&](int x, int slot) {
+        const u32x2 w = mask_words(x, slot);
+        const bool any = __builtin_amdgcn_ballot_w64((w.x | w.y) != 0u) != 0ull;
+        if (lane == 0) s_live[slot * 4 + wave] = any ? 1u : 0u;
+    };
+    auto read_live = [&](int slot) -> bool {
+        const u32x4 f = lds_read_b128(lds0 + OFF_LIVE + slot * 16);
+        return __builtin_amdgcn_readfirstlane(f.x | f.y | f.z | f.w) != 0u;
     };
 
     // ---- K/V tiles: async copies --------------------------------------------------------------
@@ -264,16 +268,6 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         }
     };
 
-    // ---- Q^T as MFMA B operands: lane holds query row l32, d = 16*s + 8*hh .. +7 (raw for now) ----
-    const int qrow = qt * BM + wave * 32 + l32;
-    u32x4 qf[4];
-#pragma unroll
-    for (int s = 0; s < 4; ++s) {
-        u32x4 t = {0u, 0u, 0u, 0u};
-        if (qrow < N) t = *reinterpret_cast<const u32x4 *>(qb + (size_t)qrow * HD + 16 * s + 8 * hh);
-        qf[s] = t;
-    }
-
     // ---- per-lane LDS read addresses (stage 0); everything else is an immediate offset ----
     // K operand (blk, s): row 32*blk + l32, chunk 2s + hh           -> kaddr[s] + 4096*blk
     // V operand (dblk, blk, u, x), read by ds_read_b64_tr_b16: the lane supplies
@@ -301,6 +295,47 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     const uint32_t lut_addr = lds0 + OFF_LUT;
     const uint32_t nib_shift = 4u - 4u * hh;
 
+    // ================================ prologue: one memory round trip ================================
+    // Everything the first two tiles need is requested at once, oldest first:
+    //   q (this wave's 32 rows, staged through the still unused third K/V stage, K-swizzled),
+    //   mask words of tiles 0..2, K/V of tile 0, K/V of tile 1.
+    const int qrow = qt * BM + wave * 32 + l32;
+    {
+        const int qbase = qt * BM + wave * 32;
+        const uint32_t dst = lds0 + 2 * STAGE_BYTES + wave * 4096;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = 8 * j + (lane >> 3);
+            const int pos = lane & 7;
+            const int grow = qbase + row < N ? qbase + row : N - 1;
+            async_copy_b128(dst + j * 1024, qb, (uint32_t)(grow * 128 + ((pos ^ ((row >> 1) & 7)) << 4)));
+        }
+    }
+    issue_mask(0, 0);
+    issue_mask(1, 1);
+    issue_mask(2, 2);
+    issue_kv(0, 0);
+    if (T > 1) issue_kv(1, 1);
+    // small LDS table for the mask: entry n (16 B) holds four floats, float j = (bit j of n) ? 0 : -inf
+    if (tid < 64)
+        reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
+
+    if (T > 1) WAIT_VMCNT(8); else WAIT_VMCNT(4);      // q and the mask words have landed
+    // ---- Q^T as MFMA B operands, scaled by scale*log2(e)/post_mul:
+    //      lane holds query row l32, d = 16*s + 8*hh .. +7
+    u32x4 qf[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        u32x4 t = lds_read_b128(kaddr[s] + 2 * STAGE_BYTES + wave * 4096);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lo = E::up1((uint16_t)(t[i] & 0xffffu)) * a.q_scale;
+            const float hi = E::up1((uint16_t)(t[i] >> 16)) * a.q_scale;
+            t[i] = (uint32_t)E::cvt1(lo) | ((uint32_t)E::cvt1(hi) << 16);
+        }
+        qf[s] = t;
+    }
+
     // ---- running state: one query row per lane; both lane halves hold the same ref ----
     f32x16 oacc[2];
 #pragma unroll
@@ -309,7 +344,8 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     float rmax = -__builtin_inff();     // largest score seen so far minus r; -inf = none yet
     float l_run = 0.f;                  // this lane's share of sum exp2(pm * (score - r))
     u32x4 refb = {0u, 0u, 0u, 0u};      // -r as four 16-bit terms (lane half 0 only), B operand
-    const u32x4 ones = {E::ONES, E::ONES, E::ONES, E::ONES};
+    u32x4 ones = {E::ONES, E::ONES, E::ONES, E::ONES};
+    asm volatile("" : "+v"(ones));      // keep the constant operand resident in registers
 
     auto set_ref = [&](float r_wanted) -> float {      // returns the value actually represented
         float rest = -r_wanted, sum = 0.f;
@@ -328,11 +364,11 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         return -sum;
     };
 
-    auto compute_tile = [&](int t, int stage) {
-        const u32x2 w2 = mask_words(t);
+    // One key tile for this wavefront.  `so` (LDS offset of the stage) is a compile-time constant
+    // in every call, so all LDS addresses below are a register plus an immediate.
+    auto compute_tile = [&](const u32x2 w2, const uint32_t so) {
         if (__builtin_amdgcn_ballot_w64((w2.x | w2.y) != 0u) == 0ull) return;
-        const uint32_t so = (uint32_t)stage * STAGE_BYTES;
-        // ---- S^T: sacc[blk][4g+j] = pm-less log2 weight of (key 32blk + 8g + 4hh + j, query l32) ----
+        // ---- S^T: sacc[blk][4g+j] = log2 weight / pm of (key 32blk + 8g + 4hh + j, query l32) ----
         f32x16 sacc[2];
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
@@ -348,13 +384,12 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         sacc[1] = E::mfma(ones, refb, sacc[1]);
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
-            const uint32_t ka = kaddr[s] + so;
-            sacc[0] = E::mfma(lds_read_b128(ka), qf[s], sacc[0]);
-            sacc[1] = E::mfma(lds_read_b128(ka + 4096), qf[s], sacc[1]);
+            sacc[0] = E::mfma(lds_read_b128(kaddr[s] + so), qf[s], sacc[0]);
+            sacc[1] = E::mfma(lds_read_b128(kaddr[s] + so + 4096), qf[s], sacc[1]);
         }
         // The matrix pipe runs an issued MFMA for 32 cycles on its own, but it is fed through the
-        // VALU issue port: a wavefront streaming VALU work would starve another one's MFMAs unless
-        // MFMA phases run at a higher wave priority than softmax phases.
+        // VALU issue port: MFMA phases run at a higher wave priority than softmax phases so that a
+        // wavefront streaming VALU work does not starve another one's MFMAs.
         __builtin_amdgcn_s_setprio(0);
         // ---- row max over this tile; move the reference only when the window is left ----
         float mx = -__builtin_inff();
@@ -403,73 +438,51 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         l_run += lsum;
         // ---- O^T += V^T * P^T : oacc[dblk][4g+j] = out(query l32, d = 32dblk + 8g + 4hh + j) ----
         __builtin_amdgcn_s_setprio(3);
-        const uint32_t va00 = vaddr[0][0] + so, va01 = vaddr[0][1] + so;
-        const uint32_t va10 = vaddr[1][0] + so, va11 = vaddr[1][1] + so;
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
                 const u32x4 pv = {pb[blk][u][0], pb[blk][u][1], pb[blk][u][2], pb[blk][u][3]};
-                const uint32_t off = 4096 * blk + 2048 * u;
-                {
-                    const u32x2 lo = lds_read_tr16_b64(va00 + off), hi = lds_read_tr16_b64(va01 + off);
+                const uint32_t off = so + 4096 * blk + 2048 * u;
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk) {
+                    const u32x2 lo = lds_read_tr16_b64(vaddr[dblk][0] + off);
+                    const u32x2 hi = lds_read_tr16_b64(vaddr[dblk][1] + off);
                     const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
-                    oacc[0] = E::mfma(va, pv, oacc[0]);
-                }
-                {
-                    const u32x2 lo = lds_read_tr16_b64(va10 + off), hi = lds_read_tr16_b64(va11 + off);
-                    const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
-                    oacc[1] = E::mfma(va, pv, oacc[1]);
+                    oacc[dblk] = E::mfma(va, pv, oacc[dblk]);
                 }
             }
     };
 
-    // ---- prologue: mask words of tiles 0..2, tile flags 0..1, K/V of tiles 0..1 ----
-    issue_mask(0);
-    issue_mask(1);
-    issue_mask(2);
-    WAIT_VMCNT(0);
-    // q was requested before the mask words, so it has arrived as well; naming its registers here
-    // makes the compiler place its own wait for them now and not after the K/V copies below.
-#pragma unroll
-    for (int s = 0; s < 4; ++s) asm volatile("" : "+v"(qf[s]));
-    __syncthreads();                       // tables and cleared flags are visible
-    mark_live(0);
-    if (T > 1) mark_live(1);
-    __syncthreads();
-    bool live0 = __builtin_amdgcn_readfirstlane(s_live[0]) != 0u;               // flag of tile t
-    bool live1 = (T > 1) && __builtin_amdgcn_readfirstlane(s_live[1]) != 0u;    // flag of tile t + 1
-    if (live0) issue_kv(0, 0);
-    if (live1) issue_kv(1, 1);
-    // scale q by scale*log2(e)/post_mul while the first tiles are in flight
-#pragma unroll
-    for (int s = 0; s < 4; ++s)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const uint32_t t = qf[s][i];
-            const float lo = E::up1((uint16_t)(t & 0xffffu)) * a.q_scale;
-            const float hi = E::up1((uint16_t)(t >> 16)) * a.q_scale;
-            qf[s][i] = (uint32_t)E::cvt1(lo) | ((uint32_t)E::cvt1(hi) << 16);
-        }
-
-    int stage = 0;
-    for (int t = 0; t < T; ++t) {
+    // ================================ main loop ================================
+    // Tile t lives in stage / mask slot t % 3; the loop is unrolled by 3 so that these are
+    // constants.  In iteration t:   wait for K/V(t) and mask(t+2)  ->  publish this wave's flag of
+    // tile t+2  ->  barrier  ->  request mask(t+3) and, if any wave flagged tile t+2, K/V(t+2)
+    // ->  compute tile t.
+    bool have0 = true;            // K/V of tile t     were requested
+    bool have1 = T > 1;           // K/V of tile t + 1 were requested
+    auto iteration = [&](const int t, auto slot_c) {
+        constexpr int SLOT = decltype(slot_c)::value;
+        constexpr int SLOT2 = (SLOT + 2) % 3;
         // copies complete in issue order: ..., K/V(t), mask(t+2), K/V(t+1)
-        if (live1) WAIT_VMCNT(4); else WAIT_VMCNT(0);
-        if (tid == 0) s_live[(t + 3) & 3] = 0u;
-        if (t + 2 < T) mark_live(t + 2);
-        if (ragged && t == T - 1 && live0) zero_tail_rows(t, stage);
-        __syncthreads();                   // K/V(t) of every wave landed; stage of tile t-1 is free
-        const bool live2 = (t + 2 < T) && __builtin_amdgcn_readfirstlane(s_live[(t + 2) & 3]) != 0u;
-        issue_mask(t + 3);
-        const int stage2 = stage == 0 ? 2 : stage - 1;             // (stage + 2) % 3
-        if (live2) issue_kv(t + 2, stage2);
-        if (live0) compute_tile(t, stage);
-        live0 = live1;
-        live1 = live2;
-        stage = stage == 2 ? 0 : stage + 1;
+        if (have1) WAIT_VMCNT(4); else WAIT_VMCNT(0);
+        const u32x2 w2 = mask_words(t, SLOT);
+        if (t + 2 < T) mark_live(t + 2, SLOT2);
+        if (ragged && t == T - 1 && have0) zero_tail_rows(t, SLOT);
+        __syncthreads();          // K/V(t) of every wave landed; the stage of tile t-1 is free
+        const bool have2 = (t + 2 < T) && read_live(SLOT2);
+        issue_mask(t + 3, SLOT);  // its words of tile t are already in w2
+        if (have2) issue_kv(t + 2, SLOT2);
+        if (have0) compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
+        have0 = have1;
+        have1 = have2;
+    };
+    for (int t = 0; t < T; t += 3) {
+        iteration(t, std::integral_constant<int, 0>{});
+        if (t + 1 < T) iteration(t + 1, std::integral_constant<int, 1>{});
+        if (t + 2 < T) iteration(t + 2, std::integral_constant<int, 2>{});
     }
-    WAIT_VMCNT(0);                          // no copy may outlive the work-group's LDS allocation
+    WAIT_VMCNT(0);                // no copy may outlive the work-group's LDS allocation
 
     // ---- epilogue ----
     const float l_tot = xhalf_sum(l_run);

@@ -18,6 +18,9 @@ from oracle import sma_oracle_c as OC
 pytestmark = pytest.mark.gpu
 
 TOL = {torch.float16: dict(atol=1e-2, rtol=1e-2), torch.bfloat16: dict(atol=1e-2, rtol=2e-2)}
+# The reference states no bar for the log-sum-exp; these follow from the rounding of the scaled
+# queries to the input format (2^-11 relative for fp16, 2^-8 for bf16).
+LSE_TOL = {torch.float16: dict(atol=2e-3, rtol=1e-3), torch.bfloat16: dict(atol=2e-2, rtol=1e-3)}
 
 
 def _run(q, k, v, mask, dev, scale=None, want_lse=False, packed=None):
@@ -80,7 +83,7 @@ def test_ragged_lengths(dev, dtype, N):
     lse_ref = O.lse_ref(q, k, mask)
     fin = torch.isfinite(lse_ref)
     assert torch.equal(torch.isfinite(lse.cpu()), fin)
-    assert torch.allclose(lse.cpu()[fin], lse_ref[fin], atol=2e-3, rtol=1e-3)
+    assert torch.allclose(lse.cpu()[fin], lse_ref[fin], **LSE_TOL[dtype])
     assert (lse.cpu()[~fin] == -math.inf).all()
 
 
