@@ -53,6 +53,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calib-copy-mib", type=int, default=0,
+                    help="also run one plain device-to-device copy of this many MiB (a traffic yardstick "
+                         "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on ONE GPU; every (b,h) pair is independent, so more "
@@ -72,6 +75,13 @@ def main():
     q, k, v, mask = harness.make_inputs(w, seed=42)
     qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
     scale = 1.0 / (w.D ** 0.5)
+
+    if args.calib_copy_mib > 0:
+        src = torch.zeros(args.calib_copy_mib << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     def step():
         packed = ext.pack_mask(md)

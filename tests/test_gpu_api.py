@@ -1,0 +1,114 @@
+"""GPU tests of the Python surface (python/sparse_attention.py over the sparse_attn_cuda module):
+same calls a user of the reference makes, checked against the oracle."""
+import importlib
+import math
+import sys
+
+import numpy as np
+import pytest
+import torch
+
+import harness
+from oracle import sma_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def sa():
+    importlib.import_module("python.sparse_attention")
+    mod = sys.modules["python.sparse_attention"]
+    assert mod.HAS_CUDA_EXT, mod._EXT_ERROR
+    return mod
+
+
+def _inputs(B, H, N, dtype, seed, keep=0.25):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = [torch.randn(B, H, N, 64, generator=g).to(dtype) for _ in range(3)]
+    mask = torch.rand(B, H, N, N, generator=g) < keep
+    return q, k, v, mask
+
+
+def test_pack_mask_returns_int32_words(sa, dev):
+    _, _, _, mask = _inputs(2, 3, 100, torch.float16, 0)
+    packed = sa.pack_mask(mask.to(dev))
+    assert packed.dtype == torch.int32 and packed.shape == (2, 3, 100, 4) and packed.is_cuda
+    assert np.array_equal(packed.cpu().numpy(), O.pack_mask_ref(mask))
+    # a non-contiguous mask (transposed view) is packed by value, like any torch op would
+    mt = mask.to(dev).transpose(-1, -2)
+    assert np.array_equal(sa.pack_mask(mt).cpu().numpy(), O.pack_mask_ref(mask.transpose(-1, -2).contiguous()))
+
+
+@pytest.mark.parametrize("fn_name", ["sparse_attention", "sparse_attention_func"])
+@pytest.mark.parametrize("dtype,rtol", [(torch.float16, 1e-2), (torch.bfloat16, 2e-2)])
+def test_forward_matches_oracle(sa, dev, fn_name, dtype, rtol):
+    q, k, v, mask = _inputs(2, 4, 256, dtype, 1)
+    mask[1, 2, 5, :] = False
+    out = getattr(sa, fn_name)(q.to(dev), k.to(dev), v.to(dev), mask.to(dev))
+    assert out.dtype == dtype and out.shape == q.shape
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    assert torch.allclose(out.float().cpu(), ref, atol=1e-2, rtol=rtol)
+    assert (out[1, 2, 5] == 0).all()
+
+
+def test_fp32_inputs_are_computed_in_bf16_and_returned_as_fp32(sa, dev):
+    """python/sparse_attention.py:140-142,151-152 of the reference."""
+    q, k, v, mask = _inputs(1, 2, 128, torch.float32, 2)
+    out = sa.sparse_attention(q.to(dev), k.to(dev), v.to(dev), mask.to(dev))
+    assert out.dtype == torch.float32
+    ref = O.sparse_attention_ref(q.bfloat16().float(), k.bfloat16().float(), v.bfloat16().float(), mask)
+    assert torch.allclose(out.cpu(), ref, atol=1e-2, rtol=2e-2)
+    assert torch.equal(out.cpu(), out.cpu().bfloat16().float())          # values are bf16 numbers
+
+
+def test_non_contiguous_inputs_and_other_stream(sa, dev):
+    q, k, v, mask = _inputs(2, 2, 192, torch.float16, 3)
+    qd = q.to(dev).transpose(1, 2).contiguous().transpose(1, 2)           # [B,H,N,D] view, strided
+    assert not qd.is_contiguous()
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        out = sa.sparse_attention_func(qd, k.to(dev), v.to(dev), mask.to(dev))
+    s.synchronize()
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    assert torch.allclose(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+
+
+def test_binding_rejects_bad_arguments(sa, dev):
+    import sparse_attn_cuda as ext
+    q, k, v, mask = _inputs(1, 1, 64, torch.float16, 4)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    packed = ext.pack_mask(md)
+    out = torch.empty_like(qd)
+    with pytest.raises(RuntimeError, match="head_dim"):
+        ext.forward(qd[..., :32].contiguous(), kd[..., :32].contiguous(), vd[..., :32].contiguous(),
+                    packed, out[..., :32].contiguous(), None, 0.125, False)
+    with pytest.raises(RuntimeError, match="Unsupported dtype"):
+        ext.forward(qd.float(), kd.float(), vd.float(), packed, out.float(), None, 0.125, False)
+    with pytest.raises(RuntimeError, match="lse"):
+        ext.forward(qd, kd, vd, packed, out, None, 0.125, True)
+    with pytest.raises(RuntimeError, match="mask_packed"):
+        ext.forward(qd, kd, vd, packed[..., :1].contiguous(), out, None, 0.125, False)
+    with pytest.raises(RuntimeError, match="bool"):
+        ext.pack_mask(md.to(torch.uint8))
+    ext.forward(qd, kd, vd, packed, out, None, 0.125, False)             # and the good call works
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()
+
+
+def test_lse_is_saved_and_backward_matches_autograd_of_the_formulation(sa, dev):
+    """.backward() of the reference raises AttributeError (sparse_attn_cuda.backward was never
+    written, python/sparse_attention.py:91-94); here it must give the gradient of the operator."""
+    q, k, v, mask = _inputs(1, 2, 96, torch.float16, 5, keep=0.4)
+    mask[0, 1, 7, :] = False
+    leaves = [t.to(dev).requires_grad_(True) for t in (q, k, v)]
+    out = sa.sparse_attention(*leaves, mask.to(dev))
+    g = torch.randn(out.shape, generator=torch.Generator().manual_seed(6)).to(torch.float16)
+    out.backward(g.to(dev))
+    ref_leaves = [t.float().requires_grad_(True) for t in (q, k, v)]
+    ref = O.sparse_attention_ref(*ref_leaves, mask)
+    ref.backward(g.float())
+    for got, want, name in zip(leaves, ref_leaves, "qkv"):
+        assert got.grad is not None and got.grad.dtype == torch.float16
+        err = (got.grad.float().cpu() - want.grad).abs().max().item()
+        assert torch.allclose(got.grad.float().cpu(), want.grad, atol=2e-2, rtol=2e-2), f"d{name} max err {err}"
+    assert (leaves[0].grad[0, 1, 7] == 0).all()
