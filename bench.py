@@ -140,7 +140,7 @@ def main():
         "roofline": {"kernel": "attn_fwd_kernel", "bound": "mfma", "achieved": round(attn_tflops, 2),
                      "peak": harness.MI355X_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(attn_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4), "traffic": None},
-        "roofline_pack": {"kernel": "pack_flat_kernel" if w.N % 32 == 0 else "pack_rows_kernel",
+        "roofline_pack": {"kernel": "pack_flat_kernel" if w.N % 32 == 0 else ("pack_row8_kernel" if w.N % 8 == 0 else "pack_rows_kernel"),
                           "bound": "hbm", "achieved": round(pack_gbps, 1), "peak": harness.MI355X_HBM_GBPS,
                           "unit": "GB/s", "frac": round(pack_gbps / harness.MI355X_HBM_GBPS, 4), "traffic": None},
     }

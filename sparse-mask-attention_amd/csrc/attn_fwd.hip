@@ -344,6 +344,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     float rmax = -__builtin_inff();     // largest score seen so far minus r; -inf = none yet
     float l_run = 0.f;                  // this lane's share of sum exp2(pm * (score - r))
     u32x4 refb = {0u, 0u, 0u, 0u};      // -r as four 16-bit terms (lane half 0 only), B operand
+    bool ref_used = false;              // false while r == 0 for every row: the extra MFMA is skipped
     u32x4 ones = {E::ONES, E::ONES, E::ONES, E::ONES};
     asm volatile("" : "+v"(ones));      // keep the constant operand resident in registers
 
@@ -380,17 +381,15 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
                 for (int j = 0; j < 4; ++j) sacc[blk][4 * g + j] = __builtin_bit_cast(float, (uint32_t)b[j]);
             }
         }
-        sacc[0] = E::mfma(ones, refb, sacc[0]);
-        sacc[1] = E::mfma(ones, refb, sacc[1]);
+        if (ref_used) {               // wave-uniform: some row of this wavefront has r != 0
+            sacc[0] = E::mfma(ones, refb, sacc[0]);
+            sacc[1] = E::mfma(ones, refb, sacc[1]);
+        }
 #pragma unroll
         for (int s = 0; s < 4; ++s) {
             sacc[0] = E::mfma(lds_read_b128(kaddr[s] + so), qf[s], sacc[0]);
             sacc[1] = E::mfma(lds_read_b128(kaddr[s] + so + 4096), qf[s], sacc[1]);
         }
-        // The matrix pipe runs an issued MFMA for 32 cycles on its own, but it is fed through the
-        // VALU issue port: MFMA phases run at a higher wave priority than softmax phases so that a
-        // wavefront streaming VALU work does not starve another one's MFMAs.
-        __builtin_amdgcn_s_setprio(0);
         // ---- row max over this tile; move the reference only when the window is left ----
         float mx = -__builtin_inff();
 #pragma unroll
@@ -409,6 +408,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
             const float delta = ref - new_ref;                       // ~ -top
             const float alpha = first ? 1.0f : __builtin_amdgcn_exp2f(POSTMUL ? delta * pm : delta);
             ref = new_ref;
+            ref_used = true;
             l_run *= alpha;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
@@ -437,7 +437,6 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
                 }
         l_run += lsum;
         // ---- O^T += V^T * P^T : oacc[dblk][4g+j] = out(query l32, d = 32dblk + 8g + 4hh + j) ----
-        __builtin_amdgcn_s_setprio(3);
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll

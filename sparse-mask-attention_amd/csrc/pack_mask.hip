@@ -9,6 +9,10 @@
 //                      (one global_load_dwordx4, fully coalesced), turns them into 16 bits, pairs up
 //                      with its neighbour lane, and even lanes store one word (coalesced 128 B per
 //                      wavefront).  Four independent spans per thread keep loads in flight.
+//   pack_row8_kernel   N % 8 == 0 (rows 8-byte aligned, e.g. N = 1000).  One wavefront per mask row:
+//                      lane l loads the 8 bytes at 8*l of a 512-byte segment (coalesced), makes 8
+//                      bits, the four lanes of a quad combine theirs with two DPP-style exchanges and
+//                      lane 4k stores word k of the segment; the last word of a row is short.
 //   pack_rows_kernel   any N.  One lane per output word, 4-byte loads when N % 4 == 0, byte loads
 //                      otherwise; the last word of a row is filled only up to column N-1.
 //
@@ -63,6 +67,39 @@ __global__ __launch_bounds__(PACK_THREADS) void pack_flat_kernel(const u32x4 *__
     }
 }
 
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+__global__ __launch_bounds__(PACK_THREADS) void pack_row8_kernel(const uint8_t *__restrict__ mask,
+                                                                 uint32_t *__restrict__ packed,
+                                                                 long long rows, int N, int nw)
+{
+    const int lane = threadIdx.x & 63;
+    const long long row = (long long)blockIdx.x * (PACK_THREADS / 64) + (threadIdx.x >> 6);
+    if (row >= rows) return;                       // whole wavefront leaves together
+    const uint8_t *src = mask + row * (long long)N;
+    uint32_t *dst = packed + row * (long long)nw;
+    for (int seg0 = 0; seg0 * 512 < N; seg0 += 4) {          // four 512-byte segments in flight
+        u32x2 d[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int col = (seg0 + u) * 512 + lane * 8;    // first column of this lane's 8 bytes
+            u32x2 x = {0u, 0u};
+            if (col < N) x = __builtin_nontemporal_load(reinterpret_cast<const u32x2 *>(src + col));
+            d[u] = x;
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            uint32_t b = __builtin_amdgcn_udot4(nonzero_bytes(d[u].x), 0x08040201u, 0u, false);
+            b = __builtin_amdgcn_udot4(nonzero_bytes(d[u].y), 0x80402010u, b, false);
+            b <<= 8 * (lane & 3);                          // position inside the word of this quad
+            b |= __shfl_xor(b, 1, 64);
+            b |= __shfl_xor(b, 2, 64);
+            const int w = (seg0 + u) * 16 + (lane >> 2);
+            if ((lane & 3) == 0 && w < nw) dst[w] = b;
+        }
+    }
+}
+
 template <bool ALIGNED4>
 __global__ __launch_bounds__(PACK_THREADS) void pack_rows_kernel(const uint8_t *__restrict__ mask,
                                                                  uint32_t *__restrict__ packed,
@@ -104,6 +141,9 @@ hipError_t launch_pack_mask(const uint8_t *mask, uint32_t *packed, long long row
         const unsigned grid = (unsigned)((n_chunks + per_block - 1) / per_block);
         hipLaunchKernelGGL(pack_flat_kernel, dim3(grid), dim3(PACK_THREADS), 0, stream,
                            reinterpret_cast<const u32x4 *>(mask), packed, n_chunks);
+    } else if ((N % 8 == 0) && ((reinterpret_cast<uintptr_t>(mask) & 7u) == 0)) {
+        const unsigned grid = (unsigned)((rows + PACK_THREADS / 64 - 1) / (PACK_THREADS / 64));
+        hipLaunchKernelGGL(pack_row8_kernel, dim3(grid), dim3(PACK_THREADS), 0, stream, mask, packed, rows, N, nw);
     } else {
         const uint32_t total = (uint32_t)(rows * nw);
         const unsigned grid = (total + PACK_THREADS - 1) / PACK_THREADS;
