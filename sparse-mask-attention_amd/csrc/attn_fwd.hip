@@ -484,10 +484,17 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     WAIT_VMCNT(0);                // no copy may outlive the work-group's LDS allocation
 
     // ---- epilogue ----
+    // out = O / l.  The accumulator layout gives a lane 8-byte pieces of one row; written as they
+    // are, a store instruction would touch 32 different 128-byte rows.  Each wave therefore
+    // transposes its 32 x 64 block through 4 KiB of LDS (K/V stage 0, free after a barrier; chunks
+    // XOR-swizzled as for K) and stores whole rows: 8 lanes x 16 B per row, 8 rows per instruction.
     const float l_tot = xhalf_sum(l_run);
     const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
-    if (qrow < N) {
-        uint16_t *ob = a.out + ((size_t)bh * N + qrow) * HD;
+    __syncthreads();              // every wave is done reading the K/V stages
+    {
+        const uint32_t obase = lds0 + wave * 4096;
+        const uint32_t wrow = obase + l32 * 128 + hh * 8;
+        const int fo = (l32 >> 1) & 7;
 #pragma unroll
         for (int dblk = 0; dblk < 2; ++dblk)
 #pragma unroll
@@ -496,9 +503,22 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
                                     ((uint32_t)E::cvt1(oacc[dblk][4 * g + 1] * inv) << 16);
                 const uint32_t hi = (uint32_t)E::cvt1(oacc[dblk][4 * g + 2] * inv) |
                                     ((uint32_t)E::cvt1(oacc[dblk][4 * g + 3] * inv) << 16);
-                u32x2 o = {lo, hi};
-                *reinterpret_cast<u32x2 *>(ob + 32 * dblk + 8 * g + 4 * hh) = o;
+                const u32x2 o = {lo, hi};
+                *(LDS_PTR(u32x2))(uintptr_t)(wrow + (((4 * dblk + g) ^ fo) << 4)) = o;
             }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        const int row0 = qt * BM + wave * 32;
+        uint16_t *ob = a.out + ((size_t)bh * N + row0) * HD;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = 8 * j + (lane >> 3), pos = lane & 7;
+            const u32x4 v = lds_read_b128(obase + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
+            if (row0 + row < N) *reinterpret_cast<u32x4 *>(ob + row * HD + pos * 8) = v;
+        }
+    }
+    if (qrow < N) {
         if (a.lse != nullptr && hh == 0) {
             // log2 of the row's sum of exp(scale * score) is pm * r + log2(l)
             a.lse[(size_t)bh * N + qrow] =
