@@ -46,6 +46,20 @@ def event_time_ms(fn, warmup, repeat, torch):
     return start.elapsed_time(end) / repeat
 
 
+def measured_traffic(kernel, workload):
+    """HBM bytes per launch from the committed rocprofv3 counter summary of this kernel and workload
+    (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a plain copy of known
+    size); None when no summary for this workload is there.  Counters cannot be read from inside
+    this process, so the figure is the recorded one, not a live one."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"{kernel}_{workload}.txt")
+    try:
+        m = re.search(r"traffic per launch ([0-9.]+) MB", open(path).read())
+    except OSError:
+        return None
+    return int(float(m.group(1)) * 1e6) if m else None
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -139,10 +153,12 @@ def main():
         "api_sparse_attention_func_ms": round(api_ms, 5),
         "roofline": {"kernel": "attn_fwd_kernel", "bound": "mfma", "achieved": round(attn_tflops, 2),
                      "peak": harness.MI355X_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(attn_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4), "traffic": None},
+                     "frac": round(attn_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4),
+                     "traffic": measured_traffic("attn_fwd_kernel", w.name), "algorithmic_bytes": w.attn_bytes},
         "roofline_pack": {"kernel": "pack_flat_kernel" if w.N % 32 == 0 else ("pack_row8_kernel" if w.N % 8 == 0 else "pack_rows_kernel"),
                           "bound": "hbm", "achieved": round(pack_gbps, 1), "peak": harness.MI355X_HBM_GBPS,
-                          "unit": "GB/s", "frac": round(pack_gbps / harness.MI355X_HBM_GBPS, 4), "traffic": None},
+                          "unit": "GB/s", "frac": round(pack_gbps / harness.MI355X_HBM_GBPS, 4),
+                          "traffic": measured_traffic("pack_mask_kernel", w.name), "algorithmic_bytes": w.pack_bytes},
     }
 
     if not args.no_cpu_baseline:
