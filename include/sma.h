@@ -70,6 +70,28 @@ int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *ma
                  void *out, float *lse, int B, int H, int N, int D, float scale, int dtype,
                  void *stream);
 
+/* Masked attention backward:  given dout = dLoss/dout, the gradients with respect to q, k and v.
+ *
+ *   dout, q, k, v, out  [B,H,N,D] fp16 or bf16 (dtype), D must be 64; out and lse are the results
+ *                       of sma_attn_fwd on the same q, k, v, mask_packed and scale
+ *   lse                 float [B,H,N] as written by sma_attn_fwd (-inf for rows that keep no key)
+ *   mask_packed         uint32 [B,H,N,ceil(N/32)]
+ *   dq, dk, dv          [B,H,N,D], same dtype; every element is written (rows that keep no key
+ *                       get dq = 0; keys that no row keeps get dk = dv = 0)
+ *   delta_ws            float [B,H,N] workspace owned by the caller; holds sum_d dout*out per query
+ *                       row on return (the library never allocates)
+ *
+ * Two launches on `stream` (dq, then dk and dv); no atomics, results are bit-reproducible.
+ *
+ * Replaces: void sparse_attention_bwd_bf16(const SparseAttentionParams&, const void* dout,
+ *           void* dq, void* dk, void* dv, cudaStream_t), declared csrc/sparse_attention.h:57-64 and
+ *           never defined; its caller is python/sparse_attention.py:91-94 and the mathematics is
+ *           the PyTorch fallback at python/sparse_attention.py:97-111.
+ */
+int sma_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                 const float *lse, const uint32_t *mask_packed, void *dq, void *dk, void *dv,
+                 float *delta_ws, int B, int H, int N, int D, float scale, int dtype, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

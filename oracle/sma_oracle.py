@@ -130,6 +130,29 @@ def lse_ref(q: torch.Tensor, k: torch.Tensor, mask: torch.Tensor,
     return torch.logsumexp(s, dim=-1)
 
 
+def sparse_attention_bwd_ref(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor,
+                             dout: torch.Tensor, scale: float | None = None):
+    """Gradients (dq, dk, dv) of sum(out * dout) for out = sparse_attention_ref(q, k, v, mask).
+
+    The closed form of the reference's PyTorch fallback, python/sparse_attention.py:97-111:
+    attn = softmax of the masked scaled scores (empty rows -> 0); dv = attn^T dout;
+    dattn = dout v^T on kept entries; ds = attn * (dattn - rowsum(dattn * attn)) * scale;
+    dq = ds k; dk = ds^T q.  Computed in the dtype given (tests pass fp32 or fp64 up-casts).
+    """
+    D = q.shape[-1]
+    if scale is None:
+        scale = 1.0 / math.sqrt(D)
+    s = torch.matmul(q, k.transpose(-2, -1)) * scale
+    s = s.masked_fill(~mask, float("-inf"))
+    attn = torch.nan_to_num(torch.softmax(s, dim=-1), nan=0.0)
+    dv = torch.matmul(attn.transpose(-2, -1), dout)
+    dattn = torch.matmul(dout, v.transpose(-2, -1)).masked_fill(~mask, 0.0)
+    ds = attn * (dattn - (dattn * attn).sum(dim=-1, keepdim=True)) * scale
+    dq = torch.matmul(ds, k)
+    dk = torch.matmul(ds.transpose(-2, -1), q)
+    return dq, dk, dv
+
+
 def attention_f64_loops(q, k, v, mask, scale: float | None = None):
     """Row-by-row float64 brute force; returns (out, lse) as float64 numpy arrays."""
     q = np.asarray(q, dtype=np.float64)

@@ -1,0 +1,498 @@
+// Masked-attention backward for gfx950 (MI355X), head_dim 64, fp16 / bf16, fp32 accumulate.
+//
+// The reference declares a backward launcher (csrc/sparse_attention.h:57-64) and its Python API
+// calls sparse_attn_cuda.backward (python/sparse_attention.py:91-94), but neither was ever
+// written; the formulas are those of its PyTorch fallback (python/sparse_attention.py:97-111):
+//
+//     P  = exp(scale * Q K^T - lse) on kept entries, 0 elsewhere      (lse saved by the forward)
+//     dV = P^T dO          dP = dO V^T          delta_i = sum_d dO_id O_id  (= sum_j P_ij dP_ij)
+//     dS = P o (dP - delta) * scale             dQ = dS K            dK = dS^T Q
+//
+// Two kernels, no atomics, bit-reproducible:
+//
+//   attn_bwd_dq_kernel   one work-group = 128 query rows, walks the key tiles exactly like the
+//                        forward: S^T = K Q^T and dP^T = V dO^T on the MFMA (lane = query row, so
+//                        lse and delta are per-lane scalars and the mask enters as the accumulator's
+//                        initial value), dS^T packed to 16 bit is the B operand of dQ^T += K^T dS^T
+//                        (K^T by transposing LDS reads).  Also writes delta to the workspace.
+//   attn_bwd_dkv_kernel  one work-group = 128 keys (lane = key), walks the query tiles:
+//                        S = Q K^T and dP = dO V^T with K, V fragments held in registers; lse and
+//                        delta of the tile's rows come from LDS (broadcast reads), the mask bit of
+//                        (row, key) is bit (key % 32) of the row's word; P and dS packed to 16 bit
+//                        are the B operands of dV^T += dO^T P and dK^T += Q^T dS.
+//
+// Tiles (64 rows x 64 x 16 bit) are copied global -> LDS by global_load_lds_dwordx4 into two
+// stages, one tile ahead; the 16-byte chunks of a row are XOR-swizzled with bitrev3((row >> 1) & 7),
+// which keeps both the row reads (ds_read_b128) and the transposing reads (ds_read_b64_tr_b16) of
+// the same tile free of bank conflicts.
+#include "attn_common.h"
+
+namespace sma {
+namespace {
+
+constexpr int HD = 64;
+constexpr int BM = 128;            // rows (queries or keys) per work-group
+constexpr int BN = 64;             // rows per streamed tile
+constexpr int NTHREADS = 256;
+constexpr int TILE_BYTES = BN * HD * 2;
+constexpr int STAGE_BYTES = 2 * TILE_BYTES;
+constexpr int NSTAGE = 2;
+constexpr int AUX_BYTES = 2048;                             // small per-tile data of a stage
+constexpr int OFF_AUX = NSTAGE * STAGE_BYTES;
+constexpr int OFF_LUT = OFF_AUX + NSTAGE * AUX_BYTES;
+constexpr int LDS_BYTES = OFF_LUT + 256;
+constexpr float LOG2E = 1.4426950408889634f;
+
+__device__ __forceinline__ int bitrev3(int f) { return ((f & 1) << 2) | (f & 2) | (f >> 2); }
+
+// Per-lane constants of the tile copies: wave w copies row blocks 2w and 2w+1 (8 rows each) of a
+// 64-row tile; lane i fills LDS chunk (row 8*blk + i/8, position i%8) with global chunk
+// position ^ bitrev3((row >> 1) & 7).
+struct TileCopy {
+    uint32_t voff[2];
+    int row[2];
+};
+__device__ __forceinline__ TileCopy make_tile_copy(int wave, int lane)
+{
+    TileCopy c;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int row = 8 * (2 * wave + j) + (lane >> 3);
+        const int pos = lane & 7;
+        c.row[j] = row;
+        c.voff[j] = (uint32_t)(row * 128 + ((pos ^ bitrev3((row >> 1) & 7)) << 4));
+    }
+    return c;
+}
+// Copy the tile whose first row is row r0 of the [N, 64] matrix `mat`; rows >= N re-read row N-1
+// (they are zeroed after landing).
+__device__ __forceinline__ void issue_tile(uint32_t dst, const uint16_t *mat, int r0, int N,
+                                           const TileCopy &c, int wave)
+{
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int over = r0 + c.row[j] - (N - 1);
+        uint32_t vo = c.voff[j];
+        if (over > 0) vo -= (uint32_t)over * 128u;
+        async_copy_b128(dst + wave * 2048 + j * 1024, mat + (size_t)r0 * HD, vo);
+    }
+}
+__device__ __forceinline__ void zero_tile_tail(uint32_t dst, int r0, int N, const TileCopy &c,
+                                               int wave, int lane)
+{
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+        if (r0 + c.row[j] >= N) {
+            const u32x4 z = {0u, 0u, 0u, 0u};
+            *(LDS_PTR(u32x4))(uintptr_t)(dst + wave * 2048 + j * 1024 + lane * 16) = z;
+        }
+}
+
+// Per-lane LDS read offsets inside a tile (add the tile's base and 4096 per block of 32 rows).
+//   rowaddr[s]       ds_read_b128: row l32, columns 16s + 8hh .. +7          (A operand, k-step s)
+//   traddr[dblk][x]  ds_read_b64_tr_b16: rows 8x + 4hh + (i >> 2) (+16u), columns 32dblk + 16G +
+//                    4(i & 3) .. +3, i = lane % 16, G = (lane % 32) / 16     (A operand = tile^T)
+struct TileRead {
+    uint32_t rowaddr[4];
+    uint32_t traddr[2][2];
+};
+__device__ __forceinline__ TileRead make_tile_read(int lane)
+{
+    TileRead r;
+    const int l32 = lane & 31, hh = lane >> 5;
+    const int fk = bitrev3((l32 >> 1) & 7);
+#pragma unroll
+    for (int s = 0; s < 4; ++s) r.rowaddr[s] = (uint32_t)(l32 * 128 + (((2 * s + hh) ^ fk) << 4));
+    const int i16 = lane & 15, G = l32 >> 4;
+    const int r3 = 4 * hh + (i16 >> 2);
+#pragma unroll
+    for (int x = 0; x < 2; ++x) {
+        const int row = 8 * x + r3;
+        const int fr = bitrev3((row >> 1) & 7);
+#pragma unroll
+        for (int dblk = 0; dblk < 2; ++dblk) {
+            const int chunk = 4 * dblk + 2 * G + ((i16 & 3) >> 1);
+            r.traddr[dblk][x] = (uint32_t)(row * 128 + ((chunk ^ fr) << 4) + ((i16 & 1) << 3));
+        }
+    }
+    return r;
+}
+
+// XCD-aware renumbering of the work-groups (the 8 XCDs take them round-robin): each XCD owns a
+// contiguous range of (b,h) pairs, so the tiles of a head are fetched into one L2 only.
+__device__ __forceinline__ int renumber_block()
+{
+    const int total = gridDim.x, bid = blockIdx.x;
+    const int xcd = bid & 7, j = bid >> 3;
+    const int base = total >> 3, rem = total & 7;
+    return xcd * base + (xcd < rem ? xcd : rem) + j;
+}
+
+// 16 bytes (8 elements) of row `row` of a [N, 64] matrix at element offset `col`.
+__device__ __forceinline__ u32x4 load_frag(const uint16_t *mat, int row, int col)
+{
+    return *reinterpret_cast<const u32x4 *>(mat + (size_t)row * HD + col);
+}
+
+// Transposed store of a 32 x 64 accumulator block (acc[dblk][4g+j] = value(row l32, column
+// 32dblk + 8g + 4hh + j)) times `mult`, through 4 KiB of wave-private LDS, as whole 128-byte rows.
+template <bool BF16>
+__device__ __forceinline__ void store_block(const f32x16 (&acc)[2], float mult, uint32_t lds_wave,
+                                            uint16_t *dst_row0, int row0, int N, int lane)
+{
+    using E = Elem<BF16>;
+    const int l32 = lane & 31, hh = lane >> 5;
+    const uint32_t wrow = lds_wave + l32 * 128 + hh * 8;
+    const int fo = (l32 >> 1) & 7;
+#pragma unroll
+    for (int dblk = 0; dblk < 2; ++dblk)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const u32x2 o = {E::pack2_rne(acc[dblk][4 * g + 0] * mult, acc[dblk][4 * g + 1] * mult),
+                             E::pack2_rne(acc[dblk][4 * g + 2] * mult, acc[dblk][4 * g + 3] * mult)};
+            *(LDS_PTR(u32x2))(uintptr_t)(wrow + (((4 * dblk + g) ^ fo) << 4)) = o;
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = 8 * j + (lane >> 3), pos = lane & 7;
+        const u32x4 v = lds_read_b128(lds_wave + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
+        if (row0 + row < N) *reinterpret_cast<u32x4 *>(dst_row0 + row * HD + pos * 8) = v;
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// ------------------------------------------------------------------------------------------------
+// dQ (and delta)
+// ------------------------------------------------------------------------------------------------
+template <bool BF16>
+__global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dq_kernel(const AttnBwdArgs a)
+{
+    using E = Elem<BF16>;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, hh = lane >> 5;
+    const int nid = renumber_block();
+    const int bh = nid / a.qtiles;
+    const int qt = nid - bh * a.qtiles;
+    const int N = a.N, nw = a.nw;
+    const int T = (N + BN - 1) / BN;
+    const bool ragged = (N & (BN - 1)) != 0;
+    const float pm = a.post_mul;
+
+    const size_t mat = (size_t)bh * N * HD;
+    const uint16_t *kb = a.k + mat, *vb = a.v + mat;
+    const uint32_t *mb = a.mask_packed + (size_t)bh * N * nw;
+
+    // ---- this lane's query row: q^T and dO^T fragments (B operands), delta, lse ----
+    const int qrow = qt * BM + wave * 32 + l32;
+    const int qr = qrow < N ? qrow : N - 1;
+    u32x4 qf[4], dof[4];
+    float delta = 0.f;
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        const int col = 16 * s + 8 * hh;
+        u32x4 tq = load_frag(a.q + mat, qr, col);
+        const u32x4 td = load_frag(a.dout + mat, qr, col);
+        const u32x4 to = load_frag(a.out + mat, qr, col);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            delta += E::up1((uint16_t)(td[i] & 0xffffu)) * E::up1((uint16_t)(to[i] & 0xffffu)) +
+                     E::up1((uint16_t)(td[i] >> 16)) * E::up1((uint16_t)(to[i] >> 16));
+            const float lo = E::up1((uint16_t)(tq[i] & 0xffffu)) * a.q_scale;
+            const float hi = E::up1((uint16_t)(tq[i] >> 16)) * a.q_scale;
+            tq[i] = (uint32_t)E::cvt1(lo) | ((uint32_t)E::cvt1(hi) << 16);
+        }
+        qf[s] = tq;
+        dof[s] = td;
+    }
+    delta = xhalf_sum(delta);
+    if (qrow < N && hh == 0) a.delta[(size_t)bh * N + qrow] = delta;
+    const float lse_row = a.lse[(size_t)bh * N + qr];
+    // p = exp2(pm * s - L); rows that kept nothing (lse = -inf) and rows beyond N get L = +inf
+    const float L = (qrow >= N || lse_row == -__builtin_inff()) ? __builtin_inff() : lse_row * LOG2E;
+
+    // ---- copies ----
+    const TileCopy tc = make_tile_copy(wave, lane);
+    const TileRead tr = make_tile_read(lane);
+    const int mrow = qt * BM + wave * 32 + (lane >> 1);
+    const uint32_t m_voff = (uint32_t)(((size_t)(mrow < N ? mrow : N - 1) * nw + (lane & 1)) * 4);
+    auto issue = [&](int t, int st) {
+        uint32_t voff = m_voff;
+        if (2 * t + 1 >= nw) voff -= (lane & 1) * 4;          // odd word count: re-read the last word
+        async_copy_b32(lds0 + OFF_AUX + st * AUX_BYTES + wave * 256, mb + 2 * t, voff);
+        issue_tile(lds0 + st * STAGE_BYTES, kb, t * BN, N, tc, wave);
+        issue_tile(lds0 + st * STAGE_BYTES + TILE_BYTES, vb, t * BN, N, tc, wave);
+    };
+    issue(0, 0);
+    if (tid < 64)
+        reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
+
+    f32x16 oacc[2];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { oacc[0][i] = 0.f; oacc[1][i] = 0.f; }
+    const uint32_t lut_addr = lds0 + OFF_LUT;
+    const uint32_t nib_shift = 4u - 4u * hh;
+
+    for (int t = 0; t < T; ++t) {
+        const int st = t & 1;
+        const uint32_t so = lds0 + st * STAGE_BYTES;
+        WAIT_VMCNT(0);
+        if (ragged && t == T - 1) {
+            zero_tile_tail(so, t * BN, N, tc, wave, lane);
+            zero_tile_tail(so + TILE_BYTES, t * BN, N, tc, wave, lane);
+        }
+        __syncthreads();          // tile t of every wave landed; the other stage is free
+        if (t + 1 < T) issue(t + 1, st ^ 1);
+
+        u32x2 w2 = lds_read_b64(lds0 + OFF_AUX + st * AUX_BYTES + wave * 256 + l32 * 8);
+        if (t == T - 1) { w2.x &= a.last_mask0; w2.y &= a.last_mask1; }
+        if (__builtin_amdgcn_ballot_w64((w2.x | w2.y) != 0u) == 0ull) continue;
+
+        // S^T (mask bias as initial value) and dP^T: element [blk][4g+j] <-> key 32blk + 8g + 4hh + j
+        f32x16 sacc[2], dacc[2];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            const uint32_t wa = (blk == 0 ? w2.x : w2.y) << nib_shift;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const u32x4 b = lds_read_b128(lut_addr + ((wa >> (8 * g)) & 0xF0u));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    sacc[blk][4 * g + j] = __builtin_bit_cast(float, (uint32_t)b[j]);
+                    dacc[blk][4 * g + j] = 0.f;
+                }
+            }
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            sacc[0] = E::mfma(lds_read_b128(tr.rowaddr[s] + so), qf[s], sacc[0]);
+            sacc[1] = E::mfma(lds_read_b128(tr.rowaddr[s] + so + 4096), qf[s], sacc[1]);
+        }
+#pragma unroll
+        for (int s = 0; s < 4; ++s) {
+            dacc[0] = E::mfma(lds_read_b128(tr.rowaddr[s] + so + TILE_BYTES), dof[s], dacc[0]);
+            dacc[1] = E::mfma(lds_read_b128(tr.rowaddr[s] + so + TILE_BYTES + 4096), dof[s], dacc[1]);
+        }
+        // dS^T / scale = P^T o (dP^T - delta), packed as B operands
+        uint32_t pb[2][2][4];
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int u = 0; u < 2; ++u)
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const int e = 8 * u + 2 * i;
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], pm, -L));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e + 1], pm, -L));
+                    pb[blk][u][i] = E::pack2_rne(p0 * (dacc[blk][e] - delta), p1 * (dacc[blk][e + 1] - delta));
+                }
+        // dQ^T += K^T dS^T
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const u32x4 pv = {pb[blk][u][0], pb[blk][u][1], pb[blk][u][2], pb[blk][u][3]};
+                const uint32_t off = so + 4096 * blk + 2048 * u;
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk) {
+                    const u32x2 lo = lds_read_tr16_b64(tr.traddr[dblk][0] + off);
+                    const u32x2 hi = lds_read_tr16_b64(tr.traddr[dblk][1] + off);
+                    const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
+                    oacc[dblk] = E::mfma(va, pv, oacc[dblk]);
+                }
+            }
+    }
+    WAIT_VMCNT(0);
+    __syncthreads();              // every wave is done reading the stages
+    const int row0 = qt * BM + wave * 32;
+    if (row0 < N)
+        store_block<BF16>(oacc, a.scale, lds0 + wave * 4096, a.dq + mat + (size_t)row0 * HD, row0, N, lane);
+}
+
+// ------------------------------------------------------------------------------------------------
+// dK and dV
+// ------------------------------------------------------------------------------------------------
+template <bool BF16>
+__global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwdArgs a)
+{
+    using E = Elem<BF16>;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31, hh = lane >> 5;
+    const int nid = renumber_block();
+    const int bh = nid / a.qtiles;
+    const int kt = nid - bh * a.qtiles;
+    const int N = a.N, nw = a.nw;
+    const int T = (N + BN - 1) / BN;
+    const bool ragged = (N & (BN - 1)) != 0;
+    const float pm = a.post_mul;
+
+    const size_t mat = (size_t)bh * N * HD;
+    const uint16_t *qb = a.q + mat, *dob = a.dout + mat;
+    const uint32_t *mb = a.mask_packed + (size_t)bh * N * nw;
+    const float *lse_b = a.lse + (size_t)bh * N, *delta_b = a.delta + (size_t)bh * N;
+
+    // ---- this lane's key: K^T (scaled) and V^T fragments, B operands ----
+    const int key0 = kt * BM + wave * 32;
+    const bool wave_valid = key0 < N;                 // wave-uniform: some key of this wave exists
+    const int key = key0 + l32;
+    const int kr = key < N ? key : N - 1;
+    const uint32_t key_ok = key < N ? 0xffffffffu : 0u;
+    const int wi = (key0 >> 5) < nw ? (key0 >> 5) : nw - 1;     // this wave's mask word of a row
+    u32x4 kf[4], vf[4];
+#pragma unroll
+    for (int s = 0; s < 4; ++s) {
+        const int col = 16 * s + 8 * hh;
+        u32x4 tk = load_frag(a.k + mat, kr, col);
+        vf[s] = load_frag(a.v + mat, kr, col);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const float lo = E::up1((uint16_t)(tk[i] & 0xffffu)) * a.q_scale;
+            const float hi = E::up1((uint16_t)(tk[i] >> 16)) * a.q_scale;
+            tk[i] = (uint32_t)E::cvt1(lo) | ((uint32_t)E::cvt1(hi) << 16);
+        }
+        kf[s] = tk;
+    }
+
+    // ---- copies: Q tile, dO tile; per wave its mask word of the 64 rows; lse (wave 0), delta (wave 1)
+    const TileCopy tc = make_tile_copy(wave, lane);
+    const TileRead tr = make_tile_read(lane);
+    auto issue = [&](int t, int st) {
+        const int r0 = t * BN;
+        const int row = r0 + lane < N ? r0 + lane : N - 1;
+        const uint32_t aux = lds0 + OFF_AUX + st * AUX_BYTES;
+        async_copy_b32(aux + wave * 256, mb + wi, (uint32_t)((size_t)row * nw * 4));
+        if (wave == 0) async_copy_b32(aux + 1024, lse_b, (uint32_t)(row * 4));
+        if (wave == 1) async_copy_b32(aux + 1280, delta_b, (uint32_t)(row * 4));
+        issue_tile(lds0 + st * STAGE_BYTES, qb, r0, N, tc, wave);
+        issue_tile(lds0 + st * STAGE_BYTES + TILE_BYTES, dob, r0, N, tc, wave);
+    };
+    issue(0, 0);
+
+    f32x16 dkacc[2], dvacc[2];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) { dkacc[0][i] = 0.f; dkacc[1][i] = 0.f; dvacc[0][i] = 0.f; dvacc[1][i] = 0.f; }
+
+    for (int t = 0; t < T; ++t) {
+        const int st = t & 1;
+        const uint32_t so = lds0 + st * STAGE_BYTES;
+        const uint32_t aux = lds0 + OFF_AUX + st * AUX_BYTES;
+        WAIT_VMCNT(0);
+        if (wave == 0) {
+            // lse of the tile's rows -> log2 units; rows that kept nothing or lie beyond N -> +inf
+            const uint32_t p = aux + 1024 + lane * 4;
+            const float l = *(LDS_PTR(float))(uintptr_t)p;
+            const bool dead = (t * BN + lane >= N) || (l == -__builtin_inff());
+            *(LDS_PTR(float))(uintptr_t)p = dead ? __builtin_inff() : l * LOG2E;
+        }
+        if (ragged && t == T - 1) {
+            zero_tile_tail(so, t * BN, N, tc, wave, lane);
+            zero_tile_tail(so + TILE_BYTES, t * BN, N, tc, wave, lane);
+        }
+        __syncthreads();
+        if (t + 1 < T) issue(t + 1, st ^ 1);
+        if (!wave_valid) continue;
+
+#pragma unroll
+        for (int blk = 0; blk < 2; ++blk) {
+            // element 4g+j of an accumulator <-> query row 32blk + 8g + 4hh + j of the tile
+            const uint32_t rsel = (uint32_t)((32 * blk + 4 * hh) * 4);
+            u32x4 mw[4];
+            uint32_t any = 0u;
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                mw[g] = lds_read_b128(aux + wave * 256 + rsel + 32 * g);
+                any |= mw[g].x | mw[g].y | mw[g].z | mw[g].w;
+            }
+            if (__builtin_amdgcn_ballot_w64((((any >> l32) & 1u) & key_ok) != 0u) == 0ull) continue;
+
+            f32x16 sacc, dacc;
+#pragma unroll
+            for (int i = 0; i < 16; ++i) { sacc[i] = 0.f; dacc[i] = 0.f; }
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                sacc = E::mfma(lds_read_b128(tr.rowaddr[s] + so + 4096 * blk), kf[s], sacc);
+#pragma unroll
+            for (int s = 0; s < 4; ++s)
+                dacc = E::mfma(lds_read_b128(tr.rowaddr[s] + so + TILE_BYTES + 4096 * blk), vf[s], dacc);
+
+            uint32_t pp[2][4], ps[2][4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+                const u32x4 Lr = lds_read_b128(aux + 1024 + rsel + 32 * g);
+                const u32x4 Dr = lds_read_b128(aux + 1280 + rsel + 32 * g);
+                float p[4], d[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)mw[g][j], (uint32_t)l32, 1u) & key_ok;
+                    const float Lj = __builtin_bit_cast(float, (uint32_t)Lr[j]);
+                    const float Dj = __builtin_bit_cast(float, (uint32_t)Dr[j]);
+                    const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[4 * g + j], pm, -Lj));
+                    p[j] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, e) & keep);
+                    d[j] = p[j] * (dacc[4 * g + j] - Dj);
+                }
+                // elements 4g .. 4g+3 are pairs (2i, 2i+1) with i = 2(g & 1), 2(g & 1) + 1 of u = g >> 1
+                pp[g >> 1][2 * (g & 1)] = E::pack2_rne(p[0], p[1]);
+                pp[g >> 1][2 * (g & 1) + 1] = E::pack2_rne(p[2], p[3]);
+                ps[g >> 1][2 * (g & 1)] = E::pack2_rne(d[0], d[1]);
+                ps[g >> 1][2 * (g & 1) + 1] = E::pack2_rne(d[2], d[3]);
+            }
+#pragma unroll
+            for (int u = 0; u < 2; ++u) {
+                const u32x4 bp = {pp[u][0], pp[u][1], pp[u][2], pp[u][3]};
+                const u32x4 bs = {ps[u][0], ps[u][1], ps[u][2], ps[u][3]};
+                const uint32_t off = so + 4096 * blk + 2048 * u;
+#pragma unroll
+                for (int dblk = 0; dblk < 2; ++dblk) {
+                    const u32x2 qlo = lds_read_tr16_b64(tr.traddr[dblk][0] + off);
+                    const u32x2 qhi = lds_read_tr16_b64(tr.traddr[dblk][1] + off);
+                    const u32x2 dlo = lds_read_tr16_b64(tr.traddr[dblk][0] + off + TILE_BYTES);
+                    const u32x2 dhi = lds_read_tr16_b64(tr.traddr[dblk][1] + off + TILE_BYTES);
+                    const u32x4 qa = {qlo.x, qlo.y, qhi.x, qhi.y};
+                    const u32x4 da = {dlo.x, dlo.y, dhi.x, dhi.y};
+                    dkacc[dblk] = E::mfma(qa, bs, dkacc[dblk]);      // dK^T += Q^T dS
+                    dvacc[dblk] = E::mfma(da, bp, dvacc[dblk]);      // dV^T += dO^T P
+                }
+            }
+        }
+    }
+    WAIT_VMCNT(0);
+    __syncthreads();
+    if (wave_valid) {
+        store_block<BF16>(dkacc, a.scale, lds0 + wave * 4096, a.dk + mat + (size_t)key0 * HD, key0, N, lane);
+        store_block<BF16>(dvacc, 1.0f, lds0 + wave * 4096, a.dv + mat + (size_t)key0 * HD, key0, N, lane);
+    }
+}
+
+}  // namespace
+
+hipError_t launch_attn_bwd(const AttnBwdArgs &a, bool bf16, hipStream_t stream)
+{
+    const long long groups = (long long)a.BH * a.qtiles;
+    if (groups == 0) return hipSuccess;
+    const dim3 grid((unsigned)groups), block(NTHREADS);
+    // dQ first: it also fills the delta workspace that the dK/dV kernel reads (same stream).
+    if (bf16) {
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<true>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<true>), grid, block, 0, stream, a);
+    } else {
+        hipLaunchKernelGGL((attn_bwd_dq_kernel<false>), grid, block, 0, stream, a);
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<false>), grid, block, 0, stream, a);
+    }
+    return hipGetLastError();
+}
+
+}  // namespace sma

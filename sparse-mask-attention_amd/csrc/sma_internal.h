@@ -23,7 +23,22 @@ struct AttnArgs {
     uint32_t last_mask0, last_mask1;   // valid-bit masks of the two mask words of the last key tile
 };
 
+// Arguments of the two backward kernels (dQ, then dK and dV), already validated.
+struct AttnBwdArgs {
+    const uint16_t *dout, *q, *k, *v, *out;   // [BH, N, 64]
+    const float *lse;                          // [BH, N] natural-log-sum-exp saved by the forward
+    const uint32_t *mask_packed;               // [BH, N, nw]
+    uint16_t *dq, *dk, *dv;                    // [BH, N, 64]
+    float *delta;                              // [BH, N] workspace: sum_d dout * out per query row
+    int BH, N, nw;
+    int qtiles;                                // ceil(N / 128)
+    float scale;                               // as given by the caller
+    float q_scale, post_mul;                   // as in AttnArgs
+    uint32_t last_mask0, last_mask1;
+};
+
 hipError_t launch_attn_fwd(const AttnArgs &a, bool bf16, hipStream_t stream);
+hipError_t launch_attn_bwd(const AttnBwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_pack_mask(const uint8_t *mask, uint32_t *packed, long long rows, int N,
                             hipStream_t stream);
 

@@ -21,8 +21,9 @@ What differs from the reference, on purpose:
   fallback would hide a broken build.  ``sparse_attention_ref`` stays available for callers who
   want the PyTorch formulation explicitly.
 * ``.backward()`` works.  The reference calls a ``sparse_attn_cuda.backward`` that was never
-  written (:91-94); here the gradient is recomputed on the GPU with PyTorch ops from the saved
-  log-sum-exp, following the reference's own formulas (:97-111).
+  written (:91-94); here that function exists (two HIP kernels, dQ and dK/dV, from the saved
+  log-sum-exp and the packed mask).  ``backward_recompute`` states the same gradients with PyTorch
+  ops (the reference's own formulas, :97-111) for cross-checks.
 """
 from __future__ import annotations
 
@@ -75,7 +76,7 @@ def sparse_attention_ref(q, k, v, mask):
 # ----------------------------------------------------------------------------------------------
 
 class SparseAttentionFunction(Function):
-    """forward = fused HIP kernel (saves LSE); backward = recomputation from LSE on the GPU."""
+    """forward = fused HIP kernel (saves LSE); backward = the HIP dQ and dK/dV kernels."""
 
     @staticmethod
     def forward(ctx, q, k, v, mask_packed, mask_bool, scale, seq_len):
@@ -85,26 +86,36 @@ class SparseAttentionFunction(Function):
         out = torch.empty_like(q)
         lse = torch.empty(B, H, N, device=q.device, dtype=torch.float32)
         sparse_attn_cuda.forward(q, k, v, mask_packed, out, lse, scale, True)
-        ctx.save_for_backward(q, k, v, out, lse, mask_bool)
+        ctx.save_for_backward(q, k, v, out, lse, mask_packed)
         ctx.scale = scale
         return out
 
     @staticmethod
     def backward(ctx, dout):
-        q, k, v, out, lse, mask_bool = ctx.saved_tensors
-        scale = ctx.scale
-        qf, kf, vf, do = q.float(), k.float(), v.float(), dout.float()
-        # p = exp(s - lse) on kept entries; rows that keep nothing have lse = -inf and p = 0.
-        s = (qf @ kf.transpose(-1, -2)) * scale
-        safe_lse = torch.where(torch.isinf(lse), torch.zeros_like(lse), lse).unsqueeze(-1)
-        p = torch.exp(s - safe_lse).masked_fill(mask_bool.logical_not(), 0.0)
-        dv = p.transpose(-1, -2) @ do
-        dp = do @ vf.transpose(-1, -2)
-        delta = (do * out.float()).sum(dim=-1, keepdim=True)      # = sum_j p_ij dp_ij
-        ds = p * (dp - delta) * scale
-        dq = ds @ kf
-        dk = ds.transpose(-1, -2) @ qf
-        return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype), None, None, None, None
+        q, k, v, out, lse, mask_packed = ctx.saved_tensors
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        # the call the reference makes at python/sparse_attention.py:91-94
+        sparse_attn_cuda.backward(dout.to(q.dtype).contiguous(), q, k, v, out, lse, mask_packed,
+                                  dq, dk, dv, ctx.scale)
+        return dq, dk, dv, None, None, None, None
+
+
+def backward_recompute(q, k, v, out, lse, mask_bool, dout, scale):
+    """The same gradients with PyTorch ops on the GPU from the saved log-sum-exp (the formulas of
+    the reference's fallback, python/sparse_attention.py:97-111).  Not used by the autograd
+    function; kept as a cross-check for users and tests."""
+    qf, kf, vf, do = q.float(), k.float(), v.float(), dout.float()
+    # p = exp(s - lse) on kept entries; rows that keep nothing have lse = -inf and p = 0.
+    s = (qf @ kf.transpose(-1, -2)) * scale
+    safe_lse = torch.where(torch.isinf(lse), torch.zeros_like(lse), lse).unsqueeze(-1)
+    p = torch.exp(s - safe_lse).masked_fill(mask_bool.logical_not(), 0.0)
+    dv = p.transpose(-1, -2) @ do
+    dp = do @ vf.transpose(-1, -2)
+    delta = (do * out.float()).sum(dim=-1, keepdim=True)      # = sum_j p_ij dp_ij
+    ds = p * (dp - delta) * scale
+    dq = ds @ kf
+    dk = ds.transpose(-1, -2) @ qf
+    return dq.to(q.dtype), dk.to(k.dtype), dv.to(v.dtype)
 
 
 # ----------------------------------------------------------------------------------------------

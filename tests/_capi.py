@@ -36,6 +36,8 @@ def load():
         lib.sma_pack_mask.argtypes = [vp, vp, ci, ci, ci, vp]
         lib.sma_attn_fwd.restype = ci
         lib.sma_attn_fwd.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_attn_bwd.restype = ci
+        lib.sma_attn_bwd.argtypes = [vp] * 11 + [ci, ci, ci, ci, cf, ci, vp]
         _lib = lib
     return _lib
 
@@ -69,3 +71,19 @@ def attn_fwd(q, k, v, packed, scale=None, want_lse=False):
                           lse.data_ptr() if want_lse else None, B, H, N, D, scale, dt, _stream())
     assert st == SMA_OK, lib.sma_strerror(st)
     return (out, lse) if want_lse else out
+
+
+def attn_bwd(dout, q, k, v, out, lse, packed, scale=None):
+    """Backward through sma_attn_bwd; returns (dq, dk, dv, delta).  Outputs are poisoned first."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    dq, dk, dv = (torch.full_like(q, float("nan")) for _ in range(3))
+    delta = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device)
+    st = lib.sma_attn_bwd(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                          lse.data_ptr(), packed.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
+                          delta.data_ptr(), B, H, N, D, scale, dt, _stream())
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return dq, dk, dv, delta

@@ -112,3 +112,48 @@ def test_lse_is_saved_and_backward_matches_autograd_of_the_formulation(sa, dev):
         err = (got.grad.float().cpu() - want.grad).abs().max().item()
         assert torch.allclose(got.grad.float().cpu(), want.grad, atol=2e-2, rtol=2e-2), f"d{name} max err {err}"
     assert (leaves[0].grad[0, 1, 7] == 0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_hip_backward_agrees_with_the_pytorch_recomputation(sa, dev, dtype):
+    """The autograd function's HIP kernels against backward_recompute (PyTorch ops on the GPU from
+    the same saved tensors); fp32 inputs go through bf16 as in the forward."""
+    q, k, v, mask = _inputs(2, 3, 200, torch.float16, 9, keep=0.3)
+    q, k, v = (t.to(dtype) for t in (q, k, v))
+    leaves = [t.to(dev).requires_grad_(True) for t in (q, k, v)]
+    md = mask.to(dev)
+    out = sa.sparse_attention(*leaves, md)
+    g = torch.randn(out.shape, generator=torch.Generator().manual_seed(10)).to(dtype).to(dev)
+    out.backward(g)
+    cdt = torch.bfloat16 if dtype == torch.float32 else dtype
+    qc, kc, vc = (t.detach().to(cdt) for t in leaves)
+    packed = sa.pack_mask(md)
+    o2 = torch.empty_like(qc)
+    lse = torch.empty(2, 3, 200, device=dev, dtype=torch.float32)
+    ext = importlib.import_module("sparse_attn_cuda")
+    ext.forward(qc, kc, vc, packed, o2, lse, 0.125, True)
+    want = sa.backward_recompute(qc, kc, vc, o2, lse, md, g.to(cdt), 0.125)
+    for got, ref, name in zip(leaves, want, "qkv"):
+        assert got.grad.dtype == dtype
+        ref = ref.float()
+        bound = 1e-4 + 1e-2 * ref.abs().max() + 2e-2 * ref.abs()
+        assert ((got.grad.float() - ref).abs() <= bound).all(), f"d{name}"
+
+
+def test_extension_backward_checks_its_arguments(sa, dev):
+    ext = importlib.import_module("sparse_attn_cuda")
+    q, k, v, mask = _inputs(1, 1, 64, torch.float16, 3)
+    qd, kd, vd = (t.to(dev) for t in (q, k, v))
+    packed = ext.pack_mask(mask.to(dev))
+    out, lse = torch.empty_like(qd), torch.empty(1, 1, 64, device=dev)
+    ext.forward(qd, kd, vd, packed, out, lse, 0.125, True)
+    dq, dk, dv = (torch.empty_like(qd) for _ in range(3))
+    with pytest.raises(RuntimeError, match="dtype"):
+        ext.backward(out.float(), qd, kd, vd, out, lse, packed, dq, dk, dv, 0.125)
+    with pytest.raises(RuntimeError, match="lse"):
+        ext.backward(out, qd, kd, vd, out, lse[..., :32], packed, dq, dk, dv, 0.125)
+    with pytest.raises(RuntimeError, match="contiguous"):
+        ext.backward(out, qd.transpose(2, 3).contiguous().transpose(2, 3), kd, vd, out, lse, packed, dq, dk, dv, 0.125)
+    ext.backward(out, qd, kd, vd, out, lse, packed, dq, dk, dv, 0.125)
+    torch.cuda.synchronize()
+    assert torch.isfinite(dq).all() and torch.isfinite(dk).all() and torch.isfinite(dv).all()

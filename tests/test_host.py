@@ -21,7 +21,7 @@ def test_library_exports_every_declared_symbol(capi):
     header = open(os.path.join(ROOT, "include", "sma.h")).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     declared = set(re.findall(r"\b(sma_[a-z_0-9]+)\s*\(", header))
-    assert {"sma_version", "sma_strerror", "sma_pack_mask", "sma_attn_fwd"} <= declared
+    assert {"sma_version", "sma_strerror", "sma_pack_mask", "sma_attn_fwd", "sma_attn_bwd"} <= declared
     for name in declared:
         assert hasattr(capi, name), f"{name} is declared in sma.h but not exported"
     assert capi.sma_version() >= 100

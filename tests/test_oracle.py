@@ -184,3 +184,58 @@ def test_lse_matches_scipy_logsumexp():
     s = (q[0, 0] @ k[0, 0].T).numpy() / 8.0
     expect = np.array([scipy.special.logsumexp(s[i][mask[0, 0, i].numpy()]) for i in range(12)])
     assert np.allclose(O.lse_ref(q, k, mask)[0, 0].numpy(), expect, atol=1e-5)
+
+
+# ---------------------------------------------------------------------------
+# backward: the closed form against automatic differentiation and finite differences
+# ---------------------------------------------------------------------------
+
+def _bwd_case(B, H, N, seed, keep=0.3, empty_row=True):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v, do = (torch.randn(B, H, N, 64, generator=g, dtype=torch.float64) for _ in range(4))
+    mask = torch.rand(B, H, N, N, generator=g) < keep
+    if empty_row and N > 2:
+        mask[:, :, 1, :] = False          # a row that keeps nothing
+        mask[:, :, :, 2] = False          # a key that nobody keeps
+    return q, k, v, do, mask
+
+
+@pytest.mark.parametrize("N", [1, 7, 33, 64])
+def test_backward_closed_form_equals_autograd(N):
+    q, k, v, do, mask = _bwd_case(2, 2, N, seed=100 + N)
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    out = O.sparse_attention_ref(qa, ka, va, mask)
+    out.backward(do)
+    dq, dk, dv = O.sparse_attention_bwd_ref(q, k, v, mask, do)
+    for got, ref in ((dq, qa.grad), (dk, ka.grad), (dv, va.grad)):
+        assert torch.allclose(got, ref, atol=1e-12, rtol=1e-10)
+    if N > 2:
+        assert (dq[:, :, 1] == 0).all()                       # empty row: no gradient to its query
+        assert (dk[:, :, 2] == 0).all() and (dv[:, :, 2] == 0).all()   # unused key: none either
+
+
+def test_backward_closed_form_equals_finite_differences():
+    q, k, v, do, mask = _bwd_case(1, 1, 5, seed=7, keep=0.6, empty_row=False)
+    scale = 0.37
+    dq, dk, dv = O.sparse_attention_bwd_ref(q, k, v, mask, do, scale=scale)
+    f = lambda q_, k_, v_: (O.sparse_attention_ref(q_, k_, v_, mask, scale=scale) * do).sum().item()
+    h = 1e-6
+    for t, grad in ((q, dq), (k, dk), (v, dv)):
+        for idx in [(0, 0, 0, 0), (0, 0, 3, 17), (0, 0, 4, 63)]:
+            tp, tm = t.clone(), t.clone()
+            tp[idx] += h
+            tm[idx] -= h
+            args_p = [tp if x is t else x for x in (q, k, v)]
+            args_m = [tm if x is t else x for x in (q, k, v)]
+            fd = (f(*args_p) - f(*args_m)) / (2 * h)
+            assert abs(fd - grad[idx].item()) < 1e-6 * max(1.0, abs(fd))
+
+
+def test_backward_all_true_mask_equals_dense_sdpa_autograd():
+    q, k, v, do, _ = _bwd_case(1, 2, 16, seed=3)
+    mask = torch.ones(1, 2, 16, 16, dtype=torch.bool)
+    qa, ka, va = (t.clone().requires_grad_(True) for t in (q, k, v))
+    torch.nn.functional.scaled_dot_product_attention(qa, ka, va).backward(do)
+    dq, dk, dv = O.sparse_attention_bwd_ref(q, k, v, mask, do)
+    for got, ref in ((dq, qa.grad), (dk, ka.grad), (dv, va.grad)):
+        assert torch.allclose(got, ref, atol=1e-10, rtol=1e-8)
