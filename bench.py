@@ -128,6 +128,14 @@ def main():
                             10, reps, torch)
     api_ms = event_time_ms(lambda: sa.sparse_attention_func(qd, kd, vd, md), 10, reps, torch)
 
+    # FLOP the kernel really executes: 32-row x 64-key blocks of the mask that hold a set bit
+    # (a wavefront skips the others), 4*32*64*D each, so that skipping is not mistaken for MFMA speed
+    Np32, Np64 = -(-w.N // 32) * 32, -(-w.N // 64) * 64
+    mp = torch.zeros(w.B, w.H, Np32, Np64, dtype=torch.bool, device=dev)
+    mp[:, :, :w.N, :w.N] = md
+    live = int(mp.view(w.B, w.H, Np32 // 32, 32, Np64 // 64, 64).any(dim=5).any(dim=3).sum().item())
+    executed_flops = live * 4 * 32 * 64 * w.D
+    del mp
     attn_tflops = w.dense_flops / (attn_ms * 1e-3) / 1e12
     pack_gbps = w.pack_bytes / (pack_ms * 1e-3) / 1e9
     result = {
@@ -149,6 +157,8 @@ def main():
         "attn_kernel_ms": round(attn_ms, 5),
         "attn_kernel_tflops": round(attn_tflops, 2),
         "attn_kernel_hbm_gbps": round(w.attn_bytes / (attn_ms * 1e-3) / 1e9, 1),
+        "attn_kernel_executed_tflops": round(executed_flops / (attn_ms * 1e-3) / 1e12, 2),
+        "attn_live_block_fraction": round(executed_flops / w.dense_flops, 4) if w.N % 64 == 0 else None,
         "pack_kernel_ms": round(pack_ms, 5),
         "api_sparse_attention_func_ms": round(api_ms, 5),
         "roofline": {"kernel": "attn_fwd_kernel", "bound": "mfma", "achieved": round(attn_tflops, 2),

@@ -122,19 +122,29 @@ def backward_recompute(q, k, v, out, lse, mask_bool, dout, scale):
 # public entry points
 # ----------------------------------------------------------------------------------------------
 
-def _check_inputs(q, k, v, mask):
+def _check_inputs(q, k, v, mask, mask_packed=None):
     assert q.shape == k.shape == v.shape, "q/k/v must have the same shape"
+    if mask_packed is not None:
+        B, H, N, _ = q.shape
+        assert mask_packed.dtype == torch.int32 and tuple(mask_packed.shape) == (B, H, N, (N + 31) // 32), \
+            "mask_packed must be the int32 [B, H, N, ceil(N/32)] result of pack_mask"
+        assert mask_packed.device == q.device, "all tensors must be on the same device"
+        return
     assert q.device == k.device == v.device == mask.device, "all tensors must be on the same device"
     assert mask.dtype == torch.bool, "mask must be a bool tensor"
 
 
-def sparse_attention(q, k, v, mask):
+def sparse_attention(q, k, v, mask, mask_packed=None):
     """Masked attention with autograd support.
 
     q, k, v: ``[B, H, N, D]`` (D = 64) bf16 / fp16 / fp32;  mask: bool ``[B, H, N, N]``, True = keep.
     Returns a tensor of q's shape and original dtype.
+
+    ``mask_packed`` (optional, not in the reference): the result of ``pack_mask(mask)`` kept from an
+    earlier call with the same mask; packing (as much HBM traffic as the attention itself at
+    N = 512) is then skipped and ``mask`` may be None.
     """
-    _check_inputs(q, k, v, mask)
+    _check_inputs(q, k, v, mask, mask_packed)
     _require_ext(q)
     B, H, N, D = q.shape
     scale = 1.0 / math.sqrt(D)
@@ -143,7 +153,8 @@ def sparse_attention(q, k, v, mask):
     if orig_dtype == torch.float32:
         q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
 
-    mask_packed = pack_mask(mask)
+    if mask_packed is None:
+        mask_packed = pack_mask(mask)
     out = SparseAttentionFunction.apply(q, k, v, mask_packed, mask, scale, N)
 
     if orig_dtype == torch.float32:
@@ -151,9 +162,9 @@ def sparse_attention(q, k, v, mask):
     return out
 
 
-def sparse_attention_func(q, k, v, mask):
+def sparse_attention_func(q, k, v, mask, mask_packed=None):
     """Inference-only variant of :func:`sparse_attention`: no autograd graph, no LSE."""
-    _check_inputs(q, k, v, mask)
+    _check_inputs(q, k, v, mask, mask_packed)
     _require_ext(q)
     D = q.shape[-1]
     scale = 1.0 / math.sqrt(D)
@@ -164,7 +175,8 @@ def sparse_attention_func(q, k, v, mask):
 
     with torch.no_grad():
         q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
-        mask_packed = pack_mask(mask)
+        if mask_packed is None:
+            mask_packed = pack_mask(mask)
         out = torch.empty_like(q)
         sparse_attn_cuda.forward(q, k, v, mask_packed, out, None, scale, False)
 

@@ -42,6 +42,12 @@ def sparse_attention_hip_fwd(q, k, v, mask):
     return out
 
 
+def sdpa_bool_mask(q, k, v, mask):
+    """PyTorch's own fused attention with the same bool mask (True = attend): the on-box
+    competitor column, as the reference compares against library kernels (run.py:514-523)."""
+    return torch.nn.functional.scaled_dot_product_attention(q, k, v, attn_mask=mask)
+
+
 def _inputs(B, H, N, seed, device):
     g = torch.Generator().manual_seed(seed)
     q, k, v = [torch.randn(B, H, N, 64, generator=g).half().to(device) for _ in range(3)]
@@ -75,12 +81,13 @@ def run_perf(device):
     peak = harness.MI355X_MFMA_F16_TFLOPS
     print("=" * 56 + f"\nperformance (fp16, H=12, D=64, sparsity 0.75; peak {peak} TFLOP/s)\n" + "=" * 56)
     print("\n[sequence length sweep]  B=16")
-    print(f"  {'N':>6}  {'latency(ms)':>12}  {'TFLOPS':>8}  {'MFU%':>7}")
+    print(f"  {'N':>6}  {'latency(ms)':>12}  {'TFLOPS':>8}  {'MFU%':>7}  {'torch SDPA(ms)':>15}  {'speed-up':>8}")
     for N in (64, 128, 256, 512, 1024):
         q, k, v, mask = _inputs(16, 12, N, 1, device)
         lat = harness.measure_latency(lambda: sparse_attention_hip_fwd(q, k, v, mask))
         tf, mfu = harness.compute_mfu(lat, 16, 12, N, 64, peak)
-        print(f"  {N:>6}  {lat:>12.4f}  {tf:>8.2f}  {mfu:>7.1f}%")
+        ref = harness.measure_latency(lambda: sdpa_bool_mask(q, k, v, mask))
+        print(f"  {N:>6}  {lat:>12.4f}  {tf:>8.2f}  {mfu:>7.1f}%  {ref:>15.4f}  {ref / lat:>7.1f}x")
     print("\n[batch size sweep]  N=512")
     print(f"  {'B':>6}  {'latency(ms)':>12}  {'TFLOPS':>8}  {'MFU%':>7}  {'seq/s':>10}")
     for B in (1, 4, 8, 16, 32, 64):

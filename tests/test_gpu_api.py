@@ -157,3 +157,15 @@ def test_extension_backward_checks_its_arguments(sa, dev):
     ext.backward(out, qd, kd, vd, out, lse, packed, dq, dk, dv, 0.125)
     torch.cuda.synchronize()
     assert torch.isfinite(dq).all() and torch.isfinite(dk).all() and torch.isfinite(dv).all()
+
+
+def test_prepacked_mask_fast_path(sa, dev):
+    q, k, v, mask = _inputs(1, 2, 130, torch.float16, 12)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    packed = sa.pack_mask(md)
+    a = sa.sparse_attention_func(qd, kd, vd, md)
+    b = sa.sparse_attention_func(qd, kd, vd, None, mask_packed=packed)
+    c = sa.sparse_attention(qd, kd, vd, None, mask_packed=packed)
+    assert torch.equal(a, b) and torch.equal(a, c)
+    with pytest.raises(AssertionError):
+        sa.sparse_attention_func(qd, kd, vd, None, mask_packed=packed[..., :2])
