@@ -33,9 +33,8 @@
 //   reference r = the online softmax does not track the exact running maximum.  r moves (and O, l
 //                 are rescaled) only when a row's scores leave the window [r-8, r+8] upwards, or
 //                 when its first finite score lies below the window; probabilities stay <= 2^8.
-//   skipping    = the work-group keeps a per-tile flag "some mask bit of my 128 rows is set",
-//                 computed two tiles ahead: tiles without it are never loaded or computed; and a
-//                 wavefront whose own 32x64 block of bits is empty skips its work for that tile.
+//   skipping    = a wavefront whose own 32 x 64 block of mask bits is empty skips its GEMMs and its
+//                 softmax for that tile (the tile itself is still copied, see the main loop).
 #include <type_traits>
 
 #include "attn_common.h"
@@ -55,8 +54,7 @@ constexpr float WINDOW_LOG2 = 8.0f;
 constexpr int STAGE_BYTES = 2 * TILE_BYTES;                 // K then V
 constexpr int OFF_MASK = NSTAGE * STAGE_BYTES;              // 3 slots x 4 waves x 64 words
 constexpr int OFF_LUT = OFF_MASK + 3 * 1024;                // 16 x 16 B
-constexpr int OFF_LIVE = OFF_LUT + 256;                     // 3 slots x 4 waves, one word each
-constexpr int LDS_BYTES = OFF_LIVE + 48;
+constexpr int LDS_BYTES = OFF_LUT + 256;
 
 template <bool BF16, bool POSTMUL>
 __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
@@ -96,11 +94,10 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     const int mrow = qt * BM + wave * 32 + (lane >> 1);
     const uint32_t m_voff = (uint32_t)(((size_t)(mrow < N ? mrow : N - 1) * nw + (lane & 1)) * 4);
     auto issue_mask = [&](int x, int slot) {
-        const int xt = x < T ? x : T - 1;
         const uint32_t dst = lds0 + OFF_MASK + slot * 1024 + wave * 256;
         uint32_t voff = m_voff;
-        if (2 * xt + 1 >= nw) voff -= (lane & 1) * 4;          // odd word count: re-read the last word
-        async_copy_b32(dst, mb + 2 * xt, voff);
+        if (2 * x + 1 >= nw) voff -= (lane & 1) * 4;           // odd word count: re-read the last word
+        async_copy_b32(dst, mb + 2 * x, voff);
     };
     const uint32_t maddr = lds0 + OFF_MASK + wave * 256 + l32 * 8;
     auto mask_words = [&](int x, int slot) -> u32x2 {
@@ -110,18 +107,6 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         w.y &= last ? a.last_mask1 : 0xffffffffu;
         return w;
     };
-    // flag "some mask bit of tile x is set in this wave's 32 rows", one word per (slot, wave)
-    uint32_t *s_live = reinterpret_cast<uint32_t *>(smem + OFF_LIVE);
-    auto mark_live = [&](int x, int slot) {
-        const u32x2 w = mask_words(x, slot);
-        const bool any = __builtin_amdgcn_ballot_w64((w.x | w.y) != 0u) != 0ull;
-        if (lane == 0) s_live[slot * 4 + wave] = any ? 1u : 0u;
-    };
-    auto read_live = [&](int slot) -> bool {
-        const u32x4 f = lds_read_b128(lds0 + OFF_LIVE + slot * 16);
-        return __builtin_amdgcn_readfirstlane(f.x | f.y | f.z | f.w) != 0u;
-    };
-
     // ---- K/V tiles: async copies --------------------------------------------------------------
     // One global_load_lds_dwordx4 fills 1 KiB = 8 tile rows.  Wave w copies row blocks 2w, 2w+1 of
     // K and of V.  Lane i fills LDS chunk (row = 8*blk + i/8, position i%8) with the global chunk
@@ -196,9 +181,8 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     const uint32_t nib_shift = 4u - 4u * hh;
 
     // ================================ prologue: one memory round trip ================================
-    // Everything the first two tiles need is requested at once, oldest first:
-    //   q (this wave's 32 rows, staged through the still unused third K/V stage, K-swizzled),
-    //   mask words of tiles 0..2, K/V of tile 0, K/V of tile 1.
+    // Requested at once, oldest first: q (this wave's 32 rows, staged through the still unused third
+    // K/V stage, K-swizzled), then the mask words and K/V of tiles 0 and 1.
     const int qrow = qt * BM + wave * 32 + l32;
     {
         const int qbase = qt * BM + wave * 32;
@@ -212,15 +196,15 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         }
     }
     issue_mask(0, 0);
-    issue_mask(1, 1);
-    issue_mask(2, 2);
     issue_kv(0, 0);
-    if (T > 1) issue_kv(1, 1);
     // small LDS table for the mask: entry n (16 B) holds four floats, float j = (bit j of n) ? 0 : -inf
     if (tid < 64)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
+    int cur = 0;                      // tile being computed
+    int n1 = T > 1 ? 1 : T;           // the following tile (T: none)
+    if (n1 < T) { issue_mask(n1, 1); issue_kv(n1, 1); }
 
-    if (T > 1) WAIT_VMCNT(8); else WAIT_VMCNT(4);      // q and the mask words have landed
+    if (n1 < T) WAIT_VMCNT(10); else WAIT_VMCNT(5);     // q has landed
     // ---- Q^T as MFMA B operands, scaled by scale*log2(e)/post_mul:
     //      lane holds query row l32, d = 16*s + 8*hh .. +7
     u32x4 qf[4];
@@ -354,32 +338,34 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     };
 
     // ================================ main loop ================================
-    // Tile t lives in stage / mask slot t % 3; the loop is unrolled by 3 so that these are
-    // constants.  In iteration t:   wait for K/V(t) and mask(t+2)  ->  publish this wave's flag of
-    // tile t+2  ->  barrier  ->  request mask(t+3) and, if any wave flagged tile t+2, K/V(t+2)
-    // ->  compute tile t.
-    bool have0 = true;            // K/V of tile t     were requested
-    bool have1 = T > 1;           // K/V of tile t + 1 were requested
-    auto iteration = [&](const int t, auto slot_c) {
+    // Tile t uses stage and mask slot t % 3; the loop is unrolled by 3 so that these are
+    // constants.  In iteration t:
+    //   wait for the copies of tile t  ->  barrier  ->  request the copies of tile t + 2 (mask
+    //   words, then K/V)  ->  compute, unless this wave's 32 x 64 block of mask bits is empty.
+    // Every tile is copied: exchanging per-tile "is any of the 128 rows live" flags between the
+    // waves (tried: through LDS two tiles ahead, and as a bit map built up front from the mask
+    // rows) cost more than the copies it saved, on block-structured masks too.
+    auto iteration = [&](auto slot_c) {
         constexpr int SLOT = decltype(slot_c)::value;
         constexpr int SLOT2 = (SLOT + 2) % 3;
-        // copies complete in issue order: ..., K/V(t), mask(t+2), K/V(t+1)
-        if (have1) WAIT_VMCNT(4); else WAIT_VMCNT(0);
-        const u32x2 w2 = mask_words(t, SLOT);
-        if (t + 2 < T) mark_live(t + 2, SLOT2);
-        if (ragged && t == T - 1 && have0) zero_tail_rows(t, SLOT);
-        __syncthreads();          // K/V(t) of every wave landed; the stage of tile t-1 is free
-        const bool have2 = (t + 2 < T) && read_live(SLOT2);
-        issue_mask(t + 3, SLOT);  // its words of tile t are already in w2
-        if (have2) issue_kv(t + 2, SLOT2);
-        if (have0) compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
-        have0 = have1;
-        have1 = have2;
+        // copies complete in issue order; only those of the next tile (5) may stay in flight
+        if (n1 < T) WAIT_VMCNT(5); else WAIT_VMCNT(0);
+        const u32x2 w2 = mask_words(cur, SLOT);
+        if (ragged && cur == T - 1) zero_tail_rows(cur, SLOT);
+        __syncthreads();          // tile t landed for every wave; the stage of tile t - 1 is free
+        const int n2 = n1 + 1 < T ? n1 + 1 : T;
+        if (n2 < T) { issue_mask(n2, SLOT2); issue_kv(n2, SLOT2); }
+        compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
+        cur = n1;
+        n1 = n2;
     };
-    for (int t = 0; t < T; t += 3) {
-        iteration(t, std::integral_constant<int, 0>{});
-        if (t + 1 < T) iteration(t + 1, std::integral_constant<int, 1>{});
-        if (t + 2 < T) iteration(t + 2, std::integral_constant<int, 2>{});
+    while (true) {
+        iteration(std::integral_constant<int, 0>{});
+        if (cur >= T) break;
+        iteration(std::integral_constant<int, 1>{});
+        if (cur >= T) break;
+        iteration(std::integral_constant<int, 2>{});
+        if (cur >= T) break;
     }
     WAIT_VMCNT(0);                // no copy may outlive the work-group's LDS allocation
 
