@@ -21,7 +21,7 @@
 //                 ds_read_b64_tr_b16 (transposing read, 8 consecutive rows x 64 B) are free of
 //                 bank conflicts on the 64-bank LDS.
 //   mask        = each wavefront copies the two packed words per query row of a tile into LDS with
-//                 one global_load_lds_dword, three tiles ahead.  A lane reads the two words of its
+//                 one global_load_lds_dword, two tiles ahead.  A lane reads the two words of its
 //                 row; each nibble selects one of 16 rows of a small LDS table of four floats that
 //                 are 0 (keep) or -inf (drop); one ds_read_b128 of that row initialises four
 //                 accumulator registers of the QK^T MFMA chain.  Masking costs no VALU work per score.

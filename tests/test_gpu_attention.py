@@ -228,3 +228,23 @@ def test_benchmark_workloads(dev, name):
     torch.cuda.synchronize()
     nonempty = md.any(dim=-1, keepdim=True).expand(-1, -1, -1, 64)
     assert torch.equal(out1.float(), nonempty.float())
+
+
+@pytest.mark.parametrize("N,dtype", [(2048, torch.float16), (4096, torch.bfloat16), (8255, torch.float16)])
+def test_long_sequences(dev, N, dtype):
+    """Many key tiles per work-group (up to 129, ragged): the ring of stages and the wait counts
+    must hold over a long loop.  One head, a banded-plus-random mask with whole empty tiles."""
+    g = torch.Generator().manual_seed(N)
+    q, k, v = [(torch.randn(1, 1, N, 64, generator=g) * 0.8).to(dtype) for _ in range(3)]
+    idx = torch.arange(N)
+    band = (idx[:, None] - idx[None, :]).abs() < 200
+    mask = (band & (torch.rand(N, N, generator=g) < 0.5)) | (torch.rand(N, N, generator=g) < 0.002)
+    mask[:, 1024:1536] = False                       # eight key tiles nobody attends to
+    mask = mask[None, None]
+    out, lse = _run(q, k, v, mask, dev, want_lse=True)
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    _assert_close(out.cpu(), ref, dtype, f"N={N}")
+    ref_lse = O.lse_ref(q, k, mask)
+    fin = torch.isfinite(ref_lse)
+    assert torch.equal(torch.isfinite(lse.cpu()), fin)
+    assert torch.allclose(lse.cpu()[fin], ref_lse[fin], **LSE_TOL[dtype])

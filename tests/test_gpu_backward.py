@@ -144,3 +144,13 @@ def test_baseline_workloads_subset(dev, name):
         _check(dq[sl], rq, w.dtype, f"{name} dq head {b},{h}")
         _check(dk[sl], rk, w.dtype, f"{name} dk head {b},{h}")
         _check(dv[sl], rv, w.dtype, f"{name} dv head {b},{h}")
+
+
+def test_long_sequence(dev):
+    N = 2304
+    g = torch.Generator().manual_seed(77)
+    q, k, v, do = ((torch.randn(1, 1, N, 64, generator=g) * 0.8).to(torch.float16) for _ in range(4))
+    idx = torch.arange(N)
+    mask = ((idx[:, None] - idx[None, :]).abs() < 150) & (torch.rand(N, N, generator=g) < 0.6)
+    mask[:, 512:768] = False
+    _compare(q, k, v, do, mask[None, None], dev, tag="N=2304")
