@@ -350,9 +350,9 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         constexpr int SLOT2 = (SLOT + 2) % 3;
         // copies complete in issue order; only those of the next tile (5) may stay in flight
         if (n1 < T) WAIT_VMCNT(5); else WAIT_VMCNT(0);
-        const u32x2 w2 = mask_words(cur, SLOT);
         if (ragged && cur == T - 1) zero_tail_rows(cur, SLOT);
         __syncthreads();          // tile t landed for every wave; the stage of tile t - 1 is free
+        const u32x2 w2 = mask_words(cur, SLOT);
         const int n2 = n1 + 1 < T ? n1 + 1 : T;
         if (n2 < T) { issue_mask(n2, SLOT2); issue_kv(n2, SLOT2); }
         compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
