@@ -27,11 +27,16 @@ def main():
     mask[0, 1, 17, :] = False                     # one query row that keeps nothing
     out = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
     lse = O.lse_ref(q, k, mask)
+    # backward: a fixed upstream gradient and the closed-form gradients of the oracle
+    import torch
+    dout = (torch.randn(q.shape, generator=torch.Generator().manual_seed(43)) * 0.5).to(q.dtype)
+    dq, dk, dv = O.sparse_attention_bwd_ref(q.float(), k.float(), v.float(), mask, dout.float())
     np.savez_compressed(
         os.path.join(os.path.dirname(os.path.abspath(__file__)), "c1_fp16.npz"),
         q=q.numpy().view(np.uint16), k=k.numpy().view(np.uint16), v=v.numpy().view(np.uint16),
         mask_bits=np.packbits(mask.numpy(), axis=-1),           # MSB-first numpy default, storage only
-        packed=O.pack_mask_ref(mask), out=out.numpy(), lse=lse.numpy())
+        packed=O.pack_mask_ref(mask), out=out.numpy(), lse=lse.numpy(),
+        dout=dout.numpy().view(np.uint16), dq=dq.numpy(), dk=dk.numpy(), dv=dv.numpy())
 
 
 if __name__ == "__main__":

@@ -30,6 +30,11 @@ def test_oracle_reproduces_the_fixture():
     fin = np.isfinite(z["lse"])
     assert np.allclose(c_lse[fin], z["lse"][fin], atol=1e-5) and (c_lse[~fin] == -np.inf).all()
     assert (~fin).sum() == 1 and (z["out"][0, 1, 17] == 0).all()
+    dout = torch.from_numpy(z["dout"].view(np.float16).copy())
+    grads = O.sparse_attention_bwd_ref(q.float(), k.float(), v.float(), mask, dout.float())
+    for got, name in zip(grads, ("dq", "dk", "dv")):
+        assert np.allclose(got.numpy(), z[name], atol=1e-6, rtol=1e-5), name
+    assert (z["dq"][0, 1, 17] == 0).all()
 
 
 @pytest.mark.gpu
@@ -45,3 +50,20 @@ def test_hip_path_matches_the_fixture(dev):
     assert np.allclose(lse.cpu().numpy()[fin], z["lse"][fin], atol=2e-3)
     assert (lse.cpu().numpy()[~fin] == -np.inf).all()
     assert (out[0, 1, 17] == 0).all()
+
+
+@pytest.mark.gpu
+def test_hip_backward_matches_the_fixture(dev):
+    import _capi
+    q, k, v, mask, z = _load()
+    dout = torch.from_numpy(z["dout"].view(np.float16).copy())
+    packed = _capi.pack_mask(mask.to(dev))
+    qd, kd, vd = q.to(dev), k.to(dev), v.to(dev)
+    out, lse = _capi.attn_fwd(qd, kd, vd, packed, want_lse=True)
+    dq, dk, dv, _ = _capi.attn_bwd(dout.to(dev), qd, kd, vd, out, lse, packed)
+    torch.cuda.synchronize()
+    for got, name in ((dq, "dq"), (dk, "dk"), (dv, "dv")):
+        ref = torch.from_numpy(z[name])
+        bound = 1e-4 + 1e-2 * ref.abs().max() + 1e-2 * ref.abs()
+        assert ((got.float().cpu() - ref).abs() <= bound).all(), name
+    assert (dq[0, 1, 17] == 0).all()
