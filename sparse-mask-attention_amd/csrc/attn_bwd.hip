@@ -170,7 +170,7 @@ __device__ __forceinline__ void store_block(const f32x16 (&acc)[2], float mult, 
 // dQ (and delta)
 // ------------------------------------------------------------------------------------------------
 template <bool BF16>
-__global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dq_kernel(const AttnBwdArgs a)
+__global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdArgs a)
 {
     using E = Elem<BF16>;
     __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
@@ -257,44 +257,37 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dq_kernel(const AttnBwdA
         if (t == T - 1) { w2.x &= a.last_mask0; w2.y &= a.last_mask1; }
         if (__builtin_amdgcn_ballot_w64((w2.x | w2.y) != 0u) == 0ull) continue;
 
-        // S^T (mask bias as initial value) and dP^T: element [blk][4g+j] <-> key 32blk + 8g + 4hh + j
-        f32x16 sacc[2], dacc[2];
+        // Per block of 32 keys: S^T (mask bias as initial value) and dP^T, element [4g+j] <-> key
+        // 32blk + 8g + 4hh + j, then dS^T / scale = P^T o (dP^T - delta), packed as B operands.
+        uint32_t pb[2][2][4];
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
+            f32x16 sacc, dacc;
             const uint32_t wa = (blk == 0 ? w2.x : w2.y) << nib_shift;
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const u32x4 b = lds_read_b128(lut_addr + ((wa >> (8 * g)) & 0xF0u));
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    sacc[blk][4 * g + j] = __builtin_bit_cast(float, (uint32_t)b[j]);
-                    dacc[blk][4 * g + j] = 0.f;
+                    sacc[4 * g + j] = __builtin_bit_cast(float, (uint32_t)b[j]);
+                    dacc[4 * g + j] = 0.f;
                 }
             }
-        }
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            sacc[0] = E::mfma(lds_read_b128(tr.rowaddr[s] + so), qf[s], sacc[0]);
-            sacc[1] = E::mfma(lds_read_b128(tr.rowaddr[s] + so + 4096), qf[s], sacc[1]);
-        }
-#pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            dacc[0] = E::mfma(lds_read_b128(tr.rowaddr[s] + so + TILE_BYTES), dof[s], dacc[0]);
-            dacc[1] = E::mfma(lds_read_b128(tr.rowaddr[s] + so + TILE_BYTES + 4096), dof[s], dacc[1]);
-        }
-        // dS^T / scale = P^T o (dP^T - delta), packed as B operands
-        uint32_t pb[2][2][4];
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
+            for (int s = 0; s < 4; ++s) {
+                sacc = E::mfma(lds_read_b128(tr.rowaddr[s] + so + 4096 * blk), qf[s], sacc);
+                dacc = E::mfma(lds_read_b128(tr.rowaddr[s] + so + TILE_BYTES + 4096 * blk), dof[s], dacc);
+            }
 #pragma unroll
             for (int u = 0; u < 2; ++u)
 #pragma unroll
                 for (int i = 0; i < 4; ++i) {
                     const int e = 8 * u + 2 * i;
-                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e], pm, -L));
-                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[blk][e + 1], pm, -L));
-                    pb[blk][u][i] = E::pack2_rne(p0 * (dacc[blk][e] - delta), p1 * (dacc[blk][e + 1] - delta));
+                    const float p0 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[e], pm, -L));
+                    const float p1 = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[e + 1], pm, -L));
+                    pb[blk][u][i] = E::pack2_rne(p0 * (dacc[e] - delta), p1 * (dacc[e + 1] - delta));
                 }
+        }
         // dQ^T += K^T dS^T
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
