@@ -200,6 +200,8 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     // small LDS table for the mask: entry n (16 B) holds four floats, float j = (bit j of n) ? 0 : -inf
     if (tid < 64)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
+    const bool even_progress = (int)blockIdx.x >= a.tail_start;
+    if (even_progress && T >= 4) __builtin_amdgcn_s_setprio(3);
     int cur = 0;                      // tile being computed
     int n1 = T > 1 ? 1 : T;           // the following tile (T: none)
     if (n1 < T) { issue_mask(n1, 1); issue_kv(n1, 1); }
@@ -348,6 +350,15 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     auto iteration = [&](auto slot_c) {
         constexpr int SLOT = decltype(slot_c)::value;
         constexpr int SLOT2 = (SLOT + 2) % 3;
+        if (even_progress) {
+            // The hardware serves the oldest wave first, so of three co-resident work-groups one
+            // finishes early and the last runs alone, at a worse rate than three together.  In the
+            // last round of work-groups, where nobody waits for the slot, a wave therefore yields
+            // as it advances.
+            if (cur == T / 4) __builtin_amdgcn_s_setprio(2);
+            else if (cur == T / 2) __builtin_amdgcn_s_setprio(1);
+            else if (cur == (3 * T) / 4) __builtin_amdgcn_s_setprio(0);
+        }
         // copies complete in issue order; only those of the next tile (5) may stay in flight
         if (n1 < T) WAIT_VMCNT(5); else WAIT_VMCNT(0);
         if (ragged && cur == T - 1) zero_tail_rows(cur, SLOT);
@@ -415,10 +426,29 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
 
 }  // namespace
 
-hipError_t launch_attn_fwd(const AttnArgs &a, bool bf16, hipStream_t stream)
+// Number of compute units of the current device (cached per device ordinal).
+static int compute_units()
 {
+    static int cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
+    if (cached[dev] == 0) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess) cached[dev] = n;
+    }
+    return cached[dev];
+}
+
+hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
+{
+    AttnArgs a = args;
     const long long groups = (long long)a.BH * a.qtiles;
     if (groups == 0) return hipSuccess;
+    // Only a grid that is resident all at once with three work-groups on (almost) every CU evens out
+    // its progress; with several rounds oldest-first is what frees slots for the waiting ones, and
+    // applying it to the last round only measured neutral.
+    const long long cus = compute_units();
+    a.tail_start = (groups > 2 * cus && groups <= 3 * cus) ? 0 : (int)groups;
     const dim3 grid((unsigned)groups), block(NTHREADS);
     const bool postmul = a.post_mul != 1.0f;
     if (bf16) {
