@@ -159,7 +159,7 @@ __device__ __forceinline__ void store_block(const f32x16 (&acc)[2], float mult, 
     for (int j = 0; j < 4; ++j) {
         const int row = 8 * j + (lane >> 3), pos = lane & 7;
         const u32x4 v = lds_read_b128(lds_wave + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
-        if (row0 + row < N) *reinterpret_cast<u32x4 *>(dst_row0 + row * HD + pos * 8) = v;
+        if (row0 + row < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst_row0 + row * HD + pos * 8));
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();

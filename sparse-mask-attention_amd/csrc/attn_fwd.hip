@@ -412,7 +412,8 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         for (int j = 0; j < 4; ++j) {
             const int row = 8 * j + (lane >> 3), pos = lane & 7;
             const u32x4 v = lds_read_b128(obase + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
-            if (row0 + row < N) *reinterpret_cast<u32x4 *>(ob + row * HD + pos * 8) = v;
+            // non-temporal: the output is not read again here and should not displace K, V and the mask
+            if (row0 + row < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(ob + row * HD + pos * 8));
         }
     }
     if (qrow < N) {
