@@ -26,9 +26,10 @@ template <> struct Elem<false> {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(f16x8, a),
                                                       __builtin_bit_cast(f16x8, b), c, 0, 0, 0);
     }
-    // Two probabilities -> one packed register (round toward zero); the row sum is taken over the
-    // SAME rounded values, so numerator and denominator stay consistent.
-    static __device__ __forceinline__ uint32_t pack2_rtz(float a, float b) {
+    // Two probabilities -> one packed register with the cheapest conversion the format has (fp16:
+    // v_cvt_pkrtz, round toward zero); the row sum is taken over the SAME rounded values, so
+    // numerator and denominator stay consistent whatever the rounding.
+    static __device__ __forceinline__ uint32_t pack2_prob(float a, float b) {
         return __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_pkrtz(a, b));
     }
     static __device__ __forceinline__ uint32_t pack2_rne(float a, float b) {     // round to nearest even
@@ -54,9 +55,10 @@ template <> struct Elem<true> {
         return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(bf16x8, a),
                                                        __builtin_bit_cast(bf16x8, b), c, 0, 0, 0);
     }
-    static __device__ __forceinline__ uint32_t pack2_rtz(float a, float b) {
-        // truncation = round toward zero for the non-negative values this is used on
-        return (__builtin_bit_cast(uint32_t, a) >> 16) | (__builtin_bit_cast(uint32_t, b) & 0xffff0000u);
+    static __device__ __forceinline__ uint32_t pack2_prob(float a, float b) {
+        // one v_cvt_pk_bf16_f32 (round to nearest even)
+        const bf16x2 h = {(__bf16)a, (__bf16)b};
+        return __builtin_bit_cast(uint32_t, h);
     }
     static __device__ __forceinline__ uint32_t pack2_rne(float a, float b) {
         const bf16x2 h = {(__bf16)a, (__bf16)b};

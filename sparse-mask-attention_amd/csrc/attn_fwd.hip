@@ -317,7 +317,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
                     const float s0 = sacc[blk][8 * u + 2 * i], s1 = sacc[blk][8 * u + 2 * i + 1];
                     const float p0 = __builtin_amdgcn_exp2f(POSTMUL ? s0 * pm : s0);
                     const float p1 = __builtin_amdgcn_exp2f(POSTMUL ? s1 * pm : s1);
-                    const uint32_t pk = E::pack2_rtz(p0, p1);
+                    const uint32_t pk = E::pack2_prob(p0, p1);
                     pb[blk][u][i] = pk;
                     lsum = E::add2(pk, lsum);
                 }
