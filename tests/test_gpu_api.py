@@ -169,3 +169,30 @@ def test_prepacked_mask_fast_path(sa, dev):
     assert torch.equal(a, b) and torch.equal(a, c)
     with pytest.raises(AssertionError):
         sa.sparse_attention_func(qd, kd, vd, None, mask_packed=packed[..., :2])
+
+
+def test_forward_can_be_captured_in_a_graph_and_replayed(sa, dev):
+    """pack_mask + forward launch on the capturing stream, allocate only through PyTorch's allocator and
+    never synchronise: a captured graph replays them; every replay is checked against an eager call."""
+    q, k, v, mask = _inputs(2, 2, 192, torch.float16, 21)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    sa.sparse_attention_func(qd, kd, vd, md)                 # warm-up outside the capture
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        sa.sparse_attention_func(qd, kd, vd, md)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = sa.sparse_attention_func(qd, kd, vd, md)
+    for rep in range(3):
+        g = torch.Generator().manual_seed(100 + rep)
+        qd.copy_(torch.randn(q.shape, generator=g).to(torch.float16))
+        md.copy_(torch.rand(mask.shape, generator=g) < 0.3)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        eager = sa.sparse_attention_func(qd, kd, vd, md)
+        torch.cuda.synchronize()
+        assert torch.equal(out_g, eager), f"replay {rep}"
