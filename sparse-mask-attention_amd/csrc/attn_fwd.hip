@@ -202,11 +202,9 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
     const bool even_progress = (int)blockIdx.x >= a.tail_start;
     if (even_progress && T >= 4) __builtin_amdgcn_s_setprio(3);
-    int cur = 0;                      // tile being computed
-    int n1 = T > 1 ? 1 : T;           // the following tile (T: none)
-    if (n1 < T) { issue_mask(n1, 1); issue_kv(n1, 1); }
+    if (T > 1) { issue_mask(1, 1); issue_kv(1, 1); }
 
-    if (n1 < T) WAIT_VMCNT(10); else WAIT_VMCNT(5);     // q has landed
+    if (T > 1) WAIT_VMCNT(10); else WAIT_VMCNT(5);       // q has landed
     // ---- Q^T as MFMA B operands, scaled by scale*log2(e)/post_mul:
     //      lane holds query row l32, d = 16*s + 8*hh .. +7
     u32x4 qf[4];
@@ -347,36 +345,29 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     // Every tile is copied: exchanging per-tile "is any of the 128 rows live" flags between the
     // waves (tried: through LDS two tiles ahead, and as a bit map built up front from the mask
     // rows) cost more than the copies it saved, on block-structured masks too.
-    auto iteration = [&](auto slot_c) {
+    auto iteration = [&](const int t, auto slot_c) {
         constexpr int SLOT = decltype(slot_c)::value;
         constexpr int SLOT2 = (SLOT + 2) % 3;
         if (even_progress) {
             // The hardware serves the oldest wave first, so of three co-resident work-groups one
-            // finishes early and the last runs alone, at a worse rate than three together.  In the
-            // last round of work-groups, where nobody waits for the slot, a wave therefore yields
-            // as it advances.
-            if (cur == T / 4) __builtin_amdgcn_s_setprio(2);
-            else if (cur == T / 2) __builtin_amdgcn_s_setprio(1);
-            else if (cur == (3 * T) / 4) __builtin_amdgcn_s_setprio(0);
+            // finishes early and the last runs alone, at a worse rate than three together.  When
+            // no other work-group waits for the slot, a wave therefore yields as it advances.
+            if (t == T / 4) __builtin_amdgcn_s_setprio(2);
+            else if (t == T / 2) __builtin_amdgcn_s_setprio(1);
+            else if (t == (3 * T) / 4) __builtin_amdgcn_s_setprio(0);
         }
         // copies complete in issue order; only those of the next tile (5) may stay in flight
-        if (n1 < T) WAIT_VMCNT(5); else WAIT_VMCNT(0);
-        if (ragged && cur == T - 1) zero_tail_rows(cur, SLOT);
+        if (t + 1 < T) WAIT_VMCNT(5); else WAIT_VMCNT(0);
+        if (ragged && t == T - 1) zero_tail_rows(t, SLOT);
         __syncthreads();          // tile t landed for every wave; the stage of tile t - 1 is free
-        const u32x2 w2 = mask_words(cur, SLOT);
-        const int n2 = n1 + 1 < T ? n1 + 1 : T;
-        if (n2 < T) { issue_mask(n2, SLOT2); issue_kv(n2, SLOT2); }
+        const u32x2 w2 = mask_words(t, SLOT);
+        if (t + 2 < T) { issue_mask(t + 2, SLOT2); issue_kv(t + 2, SLOT2); }
         compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
-        cur = n1;
-        n1 = n2;
     };
-    while (true) {
-        iteration(std::integral_constant<int, 0>{});
-        if (cur >= T) break;
-        iteration(std::integral_constant<int, 1>{});
-        if (cur >= T) break;
-        iteration(std::integral_constant<int, 2>{});
-        if (cur >= T) break;
+    for (int t = 0; t < T; t += 3) {
+        iteration(t, std::integral_constant<int, 0>{});
+        if (t + 1 < T) iteration(t + 1, std::integral_constant<int, 1>{});
+        if (t + 2 < T) iteration(t + 2, std::integral_constant<int, 2>{});
     }
     WAIT_VMCNT(0);                // no copy may outlive the work-group's LDS allocation
 

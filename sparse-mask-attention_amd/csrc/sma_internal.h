@@ -21,9 +21,9 @@ struct AttnArgs {
     float q_scale;
     float post_mul;
     uint32_t last_mask0, last_mask1;   // valid-bit masks of the two mask words of the last key tile
-    // Work-groups with a linear id >= tail_start are the last ones dispatched: no other work-group
-    // waits for their slot.  Their waves lower their priority as they advance, so that the (up to
-    // three) work-groups of a CU finish together instead of oldest first.
+    // Work-groups with a linear id >= tail_start lower their waves' priority as they advance, so
+    // that the (up to three) work-groups of a CU finish together instead of oldest first.  The
+    // launcher sets 0 when the whole grid is resident at once, else the grid size (nobody yields).
     int tail_start;
 };
 
