@@ -2,8 +2,9 @@
  *
  * Plain C, plain pointers and sizes.  Every pointer is a DEVICE pointer in the address space of
  * the GPU that is current on the calling thread; `stream` is a hipStream_t passed as void*
- * (NULL = the default stream).  All tensors are dense row-major ("contiguous").  Launches are
- * asynchronous on `stream`; the functions never synchronise, never allocate and keep no state.
+ * (NULL = the default stream).  Tensors are dense row-major ("contiguous") except in the *_strided
+ * entry points, which take explicit strides.  Launches are asynchronous on `stream`; the functions
+ * never synchronise, never allocate and keep no state.
  * Return value: SMA_OK (0) or a negative SMA_ERR_* code; sma_strerror() names it.
  *
  * Each entry point cites the interface of the reference implementation that it stands in for
@@ -26,6 +27,7 @@ extern "C" {
 #define SMA_ERR_SCALE         -5   /* scale is NaN or infinite */
 #define SMA_ERR_LAUNCH        -6   /* the HIP runtime refused the launch (hipGetLastError) */
 #define SMA_ERR_ALIGNMENT     -7   /* q/k/v/out not 16-byte aligned, or mask_packed/lse not 4-byte aligned */
+#define SMA_ERR_STRIDE        -8   /* a stride is negative, not a multiple of 8 elements, or too large */
 
 #define SMA_DTYPE_F16   0
 #define SMA_DTYPE_BF16  1
@@ -91,6 +93,45 @@ int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *ma
 int sma_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
                  const float *lse, const uint32_t *mask_packed, void *dq, void *dk, void *dv,
                  float *delta_ws, int B, int H, int N, int D, float scale, int dtype, void *stream);
+
+/* A [B,H,N,D] tensor of 16-bit elements with explicit strides, in ELEMENTS.  The D elements of a
+ * row are contiguous (stride 1, not stored).  Every stride must be >= 0 and a multiple of 8 (rows
+ * stay 16-byte aligned); stride_n < 2^23, (N-1)*stride_n*2 + 2*D < 2^31 (bytes inside one (b,h)
+ * slab) and stride_b, stride_h < 2^35.  A stride of 0 on
+ * an input repeats the same data; the rows of an output must not overlap.
+ *
+ * Replaces: the twelve stride fields of SparseAttentionParams (stride_qb .. stride_on,
+ *           csrc/sparse_attention.h:30-33), which the reference declares and never reads.
+ */
+typedef struct sma_tensor {
+    void *data;                 /* element (0,0,0,0) */
+    int64_t stride_b, stride_h, stride_n;
+} sma_tensor;
+
+/* sma_attn_fwd for strided q, k, v, out and for a mask shared between batch entries and/or heads.
+ *
+ *   mask_packed     uint32 [Bm,Hm,N,ceil(N/32)] with Bm in {1,B} and Hm in {1,H}; its rows are
+ *                   contiguous; mask_stride_b / mask_stride_h are in 32-bit WORDS, >= 0, and 0 means
+ *                   that every batch entry / head reads the same mask (a [1,1,N,N] or [B,1,N,N]
+ *                   attend-mask is then packed once, not B*H times)
+ *   lse             NULL or float [B,H,N], contiguous
+ *
+ * Everything else is as for sma_attn_fwd, which is this function with contiguous strides.
+ */
+int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_tensor *v,
+                         const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                         const sma_tensor *out, float *lse, int B, int H, int N, int D, float scale,
+                         int dtype, void *stream);
+
+/* sma_attn_bwd for strided dout, q, k, v, out, dq, dk, dv and a shared mask (see
+ * sma_attn_fwd_strided); lse and delta_ws are contiguous float [B,H,N].
+ */
+int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_tensor *k,
+                         const sma_tensor *v, const sma_tensor *out, const float *lse,
+                         const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                         const sma_tensor *dq, const sma_tensor *dk, const sma_tensor *dv,
+                         float *delta_ws, int B, int H, int N, int D, float scale, int dtype,
+                         void *stream);
 
 #ifdef __cplusplus
 }

@@ -49,7 +49,7 @@ __device__ __forceinline__ int bitrev3(int f) { return ((f & 1) << 2) | (f & 2) 
 // 64-row tile; lane i fills LDS chunk (row 8*blk + i/8, position i%8) with global chunk
 // position ^ bitrev3((row >> 1) & 7).
 struct TileCopy {
-    uint32_t voff[2];
+    uint32_t chunk[2];      // byte offset of the lane's global chunk inside its row
     int row[2];
 };
 __device__ __forceinline__ TileCopy make_tile_copy(int wave, int lane)
@@ -60,21 +60,21 @@ __device__ __forceinline__ TileCopy make_tile_copy(int wave, int lane)
         const int row = 8 * (2 * wave + j) + (lane >> 3);
         const int pos = lane & 7;
         c.row[j] = row;
-        c.voff[j] = (uint32_t)(row * 128 + ((pos ^ bitrev3((row >> 1) & 7)) << 4));
+        c.chunk[j] = (uint32_t)((pos ^ bitrev3((row >> 1) & 7)) << 4);
     }
     return c;
 }
-// Copy the tile whose first row is row r0 of the [N, 64] matrix `mat`; rows >= N re-read row N-1
-// (they are zeroed after landing).
-__device__ __forceinline__ void issue_tile(uint32_t dst, const uint16_t *mat, int r0, int N,
-                                           const TileCopy &c, int wave)
+// Copy the tile whose first row is row r0 of the N-row matrix `mat` (row stride sn elements, below
+// 2^23); rows >= N re-read row N-1 (they are zeroed after landing).
+__device__ __forceinline__ void issue_tile(uint32_t dst, const uint16_t *mat, uint32_t sn, int r0,
+                                           int N, const TileCopy &c, int wave)
 {
+    const uint16_t *src = mat + (size_t)r0 * sn;
+    const int last = N - 1 - r0;
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
-        const int over = r0 + c.row[j] - (N - 1);
-        uint32_t vo = c.voff[j];
-        if (over > 0) vo -= (uint32_t)over * 128u;
-        async_copy_b128(dst + wave * 2048 + j * 1024, mat + (size_t)r0 * HD, vo);
+        const int r = c.row[j] < last ? c.row[j] : last;
+        async_copy_b128(dst + wave * 2048 + j * 1024, src, __umul24(r, 2u * sn) + c.chunk[j]);
     }
 }
 __device__ __forceinline__ void zero_tile_tail(uint32_t dst, int r0, int N, const TileCopy &c,
@@ -128,17 +128,18 @@ __device__ __forceinline__ int renumber_block()
     return xcd * base + (xcd < rem ? xcd : rem) + j;
 }
 
-// 16 bytes (8 elements) of row `row` of a [N, 64] matrix at element offset `col`.
-__device__ __forceinline__ u32x4 load_frag(const uint16_t *mat, int row, int col)
+// 16 bytes (8 elements) of row `row` (row stride sn elements) at element offset `col`.
+__device__ __forceinline__ u32x4 load_frag(const uint16_t *mat, int sn, int row, int col)
 {
-    return *reinterpret_cast<const u32x4 *>(mat + (size_t)row * HD + col);
+    return *reinterpret_cast<const u32x4 *>(mat + (size_t)row * sn + col);
 }
 
 // Transposed store of a 32 x 64 accumulator block (acc[dblk][4g+j] = value(row l32, column
-// 32dblk + 8g + 4hh + j)) times `mult`, through 4 KiB of wave-private LDS, as whole 128-byte rows.
+// 32dblk + 8g + 4hh + j)) times `mult`, through 4 KiB of wave-private LDS, as whole 128-byte rows
+// (dst_row0: the block's first row; sn: row stride in elements).
 template <bool BF16>
 __device__ __forceinline__ void store_block(const f32x16 (&acc)[2], float mult, uint32_t lds_wave,
-                                            uint16_t *dst_row0, int row0, int N, int lane)
+                                            uint16_t *dst_row0, int sn, int row0, int N, int lane)
 {
     using E = Elem<BF16>;
     const int l32 = lane & 31, hh = lane >> 5;
@@ -159,7 +160,7 @@ __device__ __forceinline__ void store_block(const f32x16 (&acc)[2], float mult, 
     for (int j = 0; j < 4; ++j) {
         const int row = 8 * j + (lane >> 3), pos = lane & 7;
         const u32x4 v = lds_read_b128(lds_wave + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
-        if (row0 + row < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst_row0 + row * HD + pos * 8));
+        if (row0 + row < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst_row0 + (size_t)row * sn + pos * 8));
     }
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
@@ -181,16 +182,17 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdA
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, hh = lane >> 5;
     const int nid = renumber_block();
-    const int bh = nid / a.qtiles;
+    const int bh = (int)fastdiv((uint32_t)nid, a.div_qtiles);
     const int qt = nid - bh * a.qtiles;
-    const int N = a.N, nw = a.nw;
+    const int N = a.N, nw = (N + 31) >> 5;
     const int T = (N + BN - 1) / BN;
     const bool ragged = (N & (BN - 1)) != 0;
     const float pm = a.post_mul;
 
-    const size_t mat = (size_t)bh * N * HD;
-    const uint16_t *kb = a.k + mat, *vb = a.v + mat;
-    const uint32_t *mb = a.mask_packed + (size_t)bh * N * nw;
+    const int bi = (int)fastdiv((uint32_t)bh, a.div_H), hi = bh - bi * a.H;
+    const uint16_t *kb = slab(a.k, bi, hi), *vb = slab(a.v, bi, hi);
+    const uint16_t *qb = slab(a.q, bi, hi), *dob = slab(a.dout, bi, hi), *ob = slab(a.out, bi, hi);
+    const uint32_t *mb = slab(a.mask, bi, hi);
 
     // ---- this lane's query row: q^T and dO^T fragments (B operands), delta, lse ----
     const int qrow = qt * BM + wave * 32 + l32;
@@ -200,9 +202,9 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdA
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
         const int col = 16 * s + 8 * hh;
-        u32x4 tq = load_frag(a.q + mat, qr, col);
-        const u32x4 td = load_frag(a.dout + mat, qr, col);
-        const u32x4 to = load_frag(a.out + mat, qr, col);
+        u32x4 tq = load_frag(qb, a.q.sn, qr, col);
+        const u32x4 td = load_frag(dob, a.dout.sn, qr, col);
+        const u32x4 to = load_frag(ob, a.out.sn, qr, col);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             delta += E::up1((uint16_t)(td[i] & 0xffffu)) * E::up1((uint16_t)(to[i] & 0xffffu)) +
@@ -229,8 +231,8 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdA
         uint32_t voff = m_voff;
         if (2 * t + 1 >= nw) voff -= (lane & 1) * 4;          // odd word count: re-read the last word
         async_copy_b32(lds0 + OFF_AUX + st * AUX_BYTES + wave * 256, mb + 2 * t, voff);
-        issue_tile(lds0 + st * STAGE_BYTES, kb, t * BN, N, tc, wave);
-        issue_tile(lds0 + st * STAGE_BYTES + TILE_BYTES, vb, t * BN, N, tc, wave);
+        issue_tile(lds0 + st * STAGE_BYTES, kb, a.k.sn, t * BN, N, tc, wave);
+        issue_tile(lds0 + st * STAGE_BYTES + TILE_BYTES, vb, a.v.sn, t * BN, N, tc, wave);
     };
     issue(0, 0);
     if (tid < 64)
@@ -308,7 +310,8 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdA
     __syncthreads();              // every wave is done reading the stages
     const int row0 = qt * BM + wave * 32;
     if (row0 < N)
-        store_block<BF16>(oacc, a.scale, lds0 + wave * 4096, a.dq + mat + (size_t)row0 * HD, row0, N, lane);
+        store_block<BF16>(oacc, a.scale, lds0 + wave * 4096, slab(a.dq, bi, hi) + (size_t)row0 * a.dq.sn,
+                          a.dq.sn, row0, N, lane);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -326,16 +329,17 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, hh = lane >> 5;
     const int nid = renumber_block();
-    const int bh = nid / a.qtiles;
+    const int bh = (int)fastdiv((uint32_t)nid, a.div_qtiles);
     const int kt = nid - bh * a.qtiles;
-    const int N = a.N, nw = a.nw;
+    const int N = a.N, nw = (N + 31) >> 5;
     const int T = (N + BN - 1) / BN;
     const bool ragged = (N & (BN - 1)) != 0;
     const float pm = a.post_mul;
 
-    const size_t mat = (size_t)bh * N * HD;
-    const uint16_t *qb = a.q + mat, *dob = a.dout + mat;
-    const uint32_t *mb = a.mask_packed + (size_t)bh * N * nw;
+    const int bi = (int)fastdiv((uint32_t)bh, a.div_H), hi = bh - bi * a.H;
+    const uint16_t *qb = slab(a.q, bi, hi), *dob = slab(a.dout, bi, hi);
+    const uint16_t *kb = slab(a.k, bi, hi), *vb = slab(a.v, bi, hi);
+    const uint32_t *mb = slab(a.mask, bi, hi);
     const float *lse_b = a.lse + (size_t)bh * N, *delta_b = a.delta + (size_t)bh * N;
 
     // ---- this lane's key: K^T (scaled) and V^T fragments, B operands ----
@@ -349,8 +353,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
 #pragma unroll
     for (int s = 0; s < 4; ++s) {
         const int col = 16 * s + 8 * hh;
-        u32x4 tk = load_frag(a.k + mat, kr, col);
-        vf[s] = load_frag(a.v + mat, kr, col);
+        u32x4 tk = load_frag(kb, a.k.sn, kr, col);
+        vf[s] = load_frag(vb, a.v.sn, kr, col);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const float lo = E::up1((uint16_t)(tk[i] & 0xffffu)) * a.q_scale;
@@ -370,8 +374,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
         async_copy_b32(aux + wave * 256, mb + wi, (uint32_t)((size_t)row * nw * 4));
         if (wave == 0) async_copy_b32(aux + 1024, lse_b, (uint32_t)(row * 4));
         if (wave == 1) async_copy_b32(aux + 1280, delta_b, (uint32_t)(row * 4));
-        issue_tile(lds0 + st * STAGE_BYTES, qb, r0, N, tc, wave);
-        issue_tile(lds0 + st * STAGE_BYTES + TILE_BYTES, dob, r0, N, tc, wave);
+        issue_tile(lds0 + st * STAGE_BYTES, qb, a.q.sn, r0, N, tc, wave);
+        issue_tile(lds0 + st * STAGE_BYTES + TILE_BYTES, dob, a.dout.sn, r0, N, tc, wave);
     };
     issue(0, 0);
 
@@ -465,15 +469,20 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     WAIT_VMCNT(0);
     __syncthreads();
     if (wave_valid) {
-        store_block<BF16>(dkacc, a.scale, lds0 + wave * 4096, a.dk + mat + (size_t)key0 * HD, key0, N, lane);
-        store_block<BF16>(dvacc, 1.0f, lds0 + wave * 4096, a.dv + mat + (size_t)key0 * HD, key0, N, lane);
+        store_block<BF16>(dkacc, a.scale, lds0 + wave * 4096, slab(a.dk, bi, hi) + (size_t)key0 * a.dk.sn,
+                          a.dk.sn, key0, N, lane);
+        store_block<BF16>(dvacc, 1.0f, lds0 + wave * 4096, slab(a.dv, bi, hi) + (size_t)key0 * a.dv.sn,
+                          a.dv.sn, key0, N, lane);
     }
 }
 
 }  // namespace
 
-hipError_t launch_attn_bwd(const AttnBwdArgs &a, bool bf16, hipStream_t stream)
+hipError_t launch_attn_bwd(const AttnBwdArgs &args, bool bf16, hipStream_t stream)
 {
+    AttnBwdArgs a = args;
+    a.div_qtiles = make_fastdiv((uint32_t)a.qtiles);
+    a.div_H = make_fastdiv((uint32_t)a.H);
     const long long groups = (long long)a.BH * a.qtiles;
     if (groups == 0) return hipSuccess;
     const dim3 grid((unsigned)groups), block(NTHREADS);

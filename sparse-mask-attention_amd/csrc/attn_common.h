@@ -18,6 +18,12 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 #define LDS_PTR(T) __attribute__((address_space(3))) T *
 
+// First element of the (b, h) slab of a strided tensor / of the packed mask.
+__device__ __forceinline__ uint16_t *slab(const Rows &r, int b, int h) {
+    return r.p + ((size_t)b * r.sb8 + (size_t)h * r.sh8) * 8;
+}
+__device__ __forceinline__ const uint32_t *slab(const PackedMask &m, int b, int h) { return m.p + b * m.sb + h * m.sh; }
+
 template <bool BF16> struct Elem;
 
 template <> struct Elem<false> {
@@ -114,6 +120,18 @@ __device__ __forceinline__ void async_copy_b128(uint32_t lds_base, const void *b
 __device__ __forceinline__ void async_copy_b32(uint32_t lds_base, const void *base, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
                  :: "s"(lds_base), "v"(voff), "s"(base) : "memory");
+}
+// The same with the LDS address given as a scalar base plus a compile-time offset: a loop that
+// copies to many fixed places then keeps one base in a scalar register instead of one per place.
+template <int OFF>
+__device__ __forceinline__ void async_copy_b128_at(uint32_t lds_base, const void *base, uint32_t voff) {
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :: "s"(lds_base), "v"(voff), "s"(base), "n"(OFF) : "memory", "scc");
+}
+template <int OFF>
+__device__ __forceinline__ void async_copy_b32_at(uint32_t lds_base, const void *base, uint32_t voff) {
+    asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
+                 :: "s"(lds_base), "v"(voff), "s"(base), "n"(OFF) : "memory", "scc");
 }
 #define WAIT_VMCNT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
 

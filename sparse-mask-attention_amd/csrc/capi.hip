@@ -8,6 +8,27 @@ namespace {
 
 inline bool misaligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 
+inline sma_tensor dense(const void *p, int H, int N, int D)
+{
+    return sma_tensor{const_cast<void *>(p), (int64_t)H * N * D, (int64_t)N * D, (int64_t)D};
+}
+
+// Checks one strided [B,H,N,64] tensor and converts it; SMA_OK or an error code.
+int to_rows(const sma_tensor *t, int N, sma::Rows *r)
+{
+    if (t == nullptr || t->data == nullptr) return SMA_ERR_NULL_POINTER;
+    if (misaligned(t->data, 16)) return SMA_ERR_ALIGNMENT;
+    if (t->stride_b < 0 || t->stride_h < 0 || t->stride_n < 0) return SMA_ERR_STRIDE;
+    if ((t->stride_b | t->stride_h | t->stride_n) & 7) return SMA_ERR_STRIDE;
+    if ((long long)(N - 1) * t->stride_n * 2 + 128 >= (1ll << 31)) return SMA_ERR_STRIDE;
+    if (t->stride_b >= (1ll << 35) || t->stride_h >= (1ll << 35) || t->stride_n >= (1ll << 23)) return SMA_ERR_STRIDE;
+    r->p = static_cast<uint16_t *>(t->data);
+    r->sb8 = (uint32_t)(t->stride_b >> 3);
+    r->sh8 = (uint32_t)(t->stride_h >> 3);
+    r->sn = (uint32_t)t->stride_n;
+    return SMA_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -25,6 +46,7 @@ const char *sma_strerror(int code)
     case SMA_ERR_SCALE:        return "scale must be finite";
     case SMA_ERR_LAUNCH:       return "HIP kernel launch failed";
     case SMA_ERR_ALIGNMENT:    return "misaligned pointer";
+    case SMA_ERR_STRIDE:       return "bad stride: negative, not a multiple of 8 elements, or too large";
     default:                   return "unknown error code";
     }
 }
@@ -68,9 +90,12 @@ static void last_tile_masks(int N, uint32_t *m0, uint32_t *m1)
     *m1 = v1 >= 32 ? 0xffffffffu : ((1u << v1) - 1u);
 }
 
-int sma_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
-                 const float *lse, const uint32_t *mask_packed, void *dq, void *dk, void *dv,
-                 float *delta_ws, int B, int H, int N, int D, float scale, int dtype, void *stream)
+int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_tensor *k,
+                         const sma_tensor *v, const sma_tensor *out, const float *lse,
+                         const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                         const sma_tensor *dq, const sma_tensor *dk, const sma_tensor *dv,
+                         float *delta_ws, int B, int H, int N, int D, float scale, int dtype,
+                         void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
     if (D != 64) return SMA_ERR_HEAD_DIM;
@@ -78,30 +103,25 @@ int sma_attn_bwd(const void *dout, const void *q, const void *k, const void *v, 
     if (!isfinite(scale)) return SMA_ERR_SCALE;
     const long long BH = (long long)B * H;
     if (BH == 0 || N == 0) return SMA_OK;
-    if (!dout || !q || !k || !v || !out || !lse || !mask_packed || !dq || !dk || !dv || !delta_ws)
-        return SMA_ERR_NULL_POINTER;
+    if (!lse || !mask_packed || !delta_ws) return SMA_ERR_NULL_POINTER;
     const long long qtiles = (N + 127) / 128;
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
-    if (misaligned(dout, 16) || misaligned(q, 16) || misaligned(k, 16) || misaligned(v, 16) ||
-        misaligned(out, 16) || misaligned(dq, 16) || misaligned(dk, 16) || misaligned(dv, 16) ||
-        misaligned(mask_packed, 4) || misaligned(lse, 4) || misaligned(delta_ws, 4))
-        return SMA_ERR_ALIGNMENT;
+    if (misaligned(mask_packed, 4) || misaligned(lse, 4) || misaligned(delta_ws, 4)) return SMA_ERR_ALIGNMENT;
+    if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 
     sma::AttnBwdArgs a;
-    a.dout = static_cast<const uint16_t *>(dout);
-    a.q = static_cast<const uint16_t *>(q);
-    a.k = static_cast<const uint16_t *>(k);
-    a.v = static_cast<const uint16_t *>(v);
-    a.out = static_cast<const uint16_t *>(out);
+    const sma_tensor *in[8] = {dout, q, k, v, out, dq, dk, dv};
+    sma::Rows *to[8] = {&a.dout, &a.q, &a.k, &a.v, &a.out, &a.dq, &a.dk, &a.dv};
+    for (int i = 0; i < 8; ++i) {
+        const int st = to_rows(in[i], N, to[i]);
+        if (st != SMA_OK) return st;
+    }
     a.lse = lse;
-    a.mask_packed = mask_packed;
-    a.dq = static_cast<uint16_t *>(dq);
-    a.dk = static_cast<uint16_t *>(dk);
-    a.dv = static_cast<uint16_t *>(dv);
+    a.mask = sma::PackedMask{mask_packed, mask_stride_b, mask_stride_h};
     a.delta = delta_ws;
     a.BH = (int)BH;
+    a.H = H;
     a.N = N;
-    a.nw = (N + 31) / 32;
     a.qtiles = (int)qtiles;
     a.scale = scale;
     split_scale(scale, &a.q_scale, &a.post_mul);
@@ -110,9 +130,10 @@ int sma_attn_bwd(const void *dout, const void *q, const void *k, const void *v, 
     return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
 }
 
-int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *mask_packed,
-                 void *out, float *lse, int B, int H, int N, int D, float scale, int dtype,
-                 void *stream)
+int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_tensor *v,
+                         const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                         const sma_tensor *out, float *lse, int B, int H, int N, int D, float scale,
+                         int dtype, void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
     if (D != 64) return SMA_ERR_HEAD_DIM;
@@ -120,29 +141,51 @@ int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *ma
     if (!isfinite(scale)) return SMA_ERR_SCALE;
     const long long BH = (long long)B * H;
     if (BH == 0 || N == 0) return SMA_OK;
-    if (!q || !k || !v || !mask_packed || !out) return SMA_ERR_NULL_POINTER;
+    if (!mask_packed) return SMA_ERR_NULL_POINTER;
     const long long qtiles = (N + 127) / 128;
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
-    if (misaligned(q, 16) || misaligned(k, 16) || misaligned(v, 16) || misaligned(out, 16) ||
-        misaligned(mask_packed, 4) || (lse && misaligned(lse, 4)))
-        return SMA_ERR_ALIGNMENT;
+    if (misaligned(mask_packed, 4) || (lse && misaligned(lse, 4))) return SMA_ERR_ALIGNMENT;
+    if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 
     sma::AttnArgs a;
-    a.q = static_cast<const uint16_t *>(q);
-    a.k = static_cast<const uint16_t *>(k);
-    a.v = static_cast<const uint16_t *>(v);
-    a.mask_packed = mask_packed;
-    a.out = static_cast<uint16_t *>(out);
+    const sma_tensor *in[4] = {q, k, v, out};
+    sma::Rows *to[4] = {&a.q, &a.k, &a.v, &a.out};
+    for (int i = 0; i < 4; ++i) {
+        const int st = to_rows(in[i], N, to[i]);
+        if (st != SMA_OK) return st;
+    }
+    a.mask = sma::PackedMask{mask_packed, mask_stride_b, mask_stride_h};
     a.lse = lse;
     a.BH = (int)BH;
+    a.H = H;
     a.N = N;
-    a.nw = (N + 31) / 32;
     a.qtiles = (int)qtiles;
     split_scale(scale, &a.q_scale, &a.post_mul);
     last_tile_masks(N, &a.last_mask0, &a.last_mask1);
 
     const hipError_t e = sma::launch_attn_fwd(a, dtype == SMA_DTYPE_BF16, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
+}
+
+int sma_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                 const float *lse, const uint32_t *mask_packed, void *dq, void *dk, void *dv,
+                 float *delta_ws, int B, int H, int N, int D, float scale, int dtype, void *stream)
+{
+    const sma_tensor t[8] = {dense(dout, H, N, D), dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D),
+                             dense(out, H, N, D), dense(dq, H, N, D), dense(dk, H, N, D), dense(dv, H, N, D)};
+    const int64_t msh = (int64_t)N * ((N + 31) / 32);
+    return sma_attn_bwd_strided(&t[0], &t[1], &t[2], &t[3], &t[4], lse, mask_packed, msh * H, msh,
+                                &t[5], &t[6], &t[7], delta_ws, B, H, N, D, scale, dtype, stream);
+}
+
+int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *mask_packed,
+                 void *out, float *lse, int B, int H, int N, int D, float scale, int dtype,
+                 void *stream)
+{
+    const sma_tensor t[4] = {dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D), dense(out, H, N, D)};
+    const int64_t msh = (int64_t)N * ((N + 31) / 32);
+    return sma_attn_fwd_strided(&t[0], &t[1], &t[2], mask_packed, msh * H, msh, &t[3], lse, B, H, N, D,
+                                scale, dtype, stream);
 }
 
 }  // extern "C"

@@ -7,14 +7,51 @@
 
 namespace sma {
 
+// A [B, H, N, 64] tensor of 16-bit elements (fp16 or bf16 bit patterns).  The 64 elements of a row
+// are contiguous; the other extents have strides that are multiples of 8 elements (rows stay
+// 16-byte aligned).  Byte offsets inside one (b, h) slab fit 31 bits (checked by the C-ABI layer).
+// Kept small: kernel arguments are fetched by every work-group before it can request any data.
+struct Rows {
+    uint16_t *p;
+    uint32_t sb8, sh8;              // batch and head strides in units of 8 elements (16 bytes)
+    uint32_t sn;                    // row stride in elements
+};
+
+// The packed mask [Bm, Hm, N, nw] with Bm in {1, B}, Hm in {1, H}: rows are contiguous, a stride of
+// 0 (in words) repeats the same mask for every batch entry / head.
+struct PackedMask {
+    const uint32_t *p;
+    long long sb, sh;
+};
+
+// Division of a work-group number by a launch constant without the (long, VALU) division sequence:
+// n / d == (n * mul) >> shift in 64-bit arithmetic for every 0 <= n < 2^31, with
+// shift = 31 + ceil(log2 d) and mul = ceil(2^shift / d) < 2^32 (round-up method: mul * d exceeds
+// 2^shift by at most 2^(shift - 31), which cannot carry into the quotient while n < 2^31).
+struct FastDiv {
+    uint32_t mul, shift;
+};
+inline FastDiv make_fastdiv(uint32_t d)
+{
+    uint32_t l = 0;
+    while ((1ull << l) < d) ++l;
+    const uint64_t p = 1ull << (31 + l);
+    return FastDiv{(uint32_t)((p + d - 1) / d), 31 + l};
+}
+__host__ __device__ inline uint32_t fastdiv(uint32_t n, FastDiv f)
+{
+    return (uint32_t)(((uint64_t)n * f.mul) >> f.shift);
+}
+
 // Arguments of the fused forward kernel, already validated by the C-ABI layer.
 struct AttnArgs {
-    const uint16_t *q, *k, *v;      // [BH, N, 64] 16-bit elements (fp16 or bf16 bit patterns)
-    const uint32_t *mask_packed;    // [BH, N, nw]
-    uint16_t *out;                  // [BH, N, 64]
-    float *lse;                     // [BH, N] or nullptr
-    int BH, N, nw;
+    Rows q, k, v;                   // inputs (never written)
+    PackedMask mask;
+    Rows out;
+    float *lse;                     // [BH, N] contiguous, or nullptr
+    int BH, H, N;
     int qtiles;                     // ceil(N / 128): query tiles (work-groups) per (b,h)
+    FastDiv div_qtiles, div_H;      // filled in by the launcher
     // exp(scale * s) is evaluated as exp2(post_mul * (q_scale * q) . k): q is multiplied by
     // q_scale (sign of scale included, |q_scale| <= 1) when it is loaded, post_mul is a power of
     // two that is 1 unless |scale| * log2(e) > 1.
@@ -29,13 +66,14 @@ struct AttnArgs {
 
 // Arguments of the two backward kernels (dQ, then dK and dV), already validated.
 struct AttnBwdArgs {
-    const uint16_t *dout, *q, *k, *v, *out;   // [BH, N, 64]
+    Rows dout, q, k, v, out;                   // inputs (never written)
     const float *lse;                          // [BH, N] natural-log-sum-exp saved by the forward
-    const uint32_t *mask_packed;               // [BH, N, nw]
-    uint16_t *dq, *dk, *dv;                    // [BH, N, 64]
+    PackedMask mask;
+    Rows dq, dk, dv;
     float *delta;                              // [BH, N] workspace: sum_d dout * out per query row
-    int BH, N, nw;
+    int BH, H, N;
     int qtiles;                                // ceil(N / 128)
+    FastDiv div_qtiles, div_H;                 // filled in by the launcher
     float scale;                               // as given by the caller
     float q_scale, post_mul;                   // as in AttnArgs
     uint32_t last_mask0, last_mask1;

@@ -15,10 +15,22 @@ SMA_ERR_DTYPE = -4
 SMA_ERR_SCALE = -5
 SMA_ERR_LAUNCH = -6
 SMA_ERR_ALIGNMENT = -7
+SMA_ERR_STRIDE = -8
 SMA_DTYPE_F16 = 0
 SMA_DTYPE_BF16 = 1
 
 _lib = None
+
+
+class SmaTensor(ctypes.Structure):
+    """struct sma_tensor of include/sma.h."""
+    _fields_ = [("data", ctypes.c_void_p), ("stride_b", ctypes.c_int64), ("stride_h", ctypes.c_int64),
+                ("stride_n", ctypes.c_int64)]
+
+    @classmethod
+    def of(cls, t: torch.Tensor) -> "SmaTensor":
+        assert t.dim() == 4 and t.stride(3) == 1
+        return cls(t.data_ptr(), t.stride(0), t.stride(1), t.stride(2))
 
 
 def load():
@@ -38,6 +50,11 @@ def load():
         lib.sma_attn_fwd.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_bwd.restype = ci
         lib.sma_attn_bwd.argtypes = [vp] * 11 + [ci, ci, ci, ci, cf, ci, vp]
+        tp, i64 = ctypes.POINTER(SmaTensor), ctypes.c_int64
+        lib.sma_attn_fwd_strided.restype = ci
+        lib.sma_attn_fwd_strided.argtypes = [tp, tp, tp, vp, i64, i64, tp, vp, ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_attn_bwd_strided.restype = ci
+        lib.sma_attn_bwd_strided.argtypes = [tp] * 5 + [vp, vp, i64, i64, tp, tp, tp, vp, ci, ci, ci, ci, cf, ci, vp]
         _lib = lib
     return _lib
 
@@ -85,5 +102,51 @@ def attn_bwd(dout, q, k, v, out, lse, packed, scale=None):
     st = lib.sma_attn_bwd(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
                           lse.data_ptr(), packed.data_ptr(), dq.data_ptr(), dk.data_ptr(), dv.data_ptr(),
                           delta.data_ptr(), B, H, N, D, scale, dt, _stream())
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return dq, dk, dv, delta
+
+
+def _mask_strides(packed, B, H):
+    """Word strides of a packed mask [Bm,Hm,N,nw] with Bm in {1,B}, Hm in {1,H}; 0 = shared."""
+    Bm, Hm, N, nw = packed.shape
+    assert Bm in (1, B) and Hm in (1, H) and packed.is_contiguous()
+    return (Hm * N * nw if Bm == B and B > 1 else 0), (N * nw if Hm == H and H > 1 else 0)
+
+
+def attn_fwd_strided(q, k, v, packed, out=None, scale=None, want_lse=False):
+    """Forward through sma_attn_fwd_strided: q, k, v (and out, if given) may be any views whose last
+    dimension is contiguous; packed may be [1|B, 1|H, N, nw]."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    if out is None:
+        out = torch.full((B, H, N, D), float("nan"), dtype=q.dtype, device=q.device)
+    lse = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device) if want_lse else None
+    msb, msh = _mask_strides(packed, B, H)
+    tq, tk, tv, to = (SmaTensor.of(t) for t in (q, k, v, out))
+    st = lib.sma_attn_fwd_strided(tq, tk, tv, packed.data_ptr(), msb, msh, to,
+                                  lse.data_ptr() if want_lse else None, B, H, N, D, scale, dt, _stream())
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return (out, lse) if want_lse else out
+
+
+def attn_bwd_strided(dout, q, k, v, out, lse, packed, grads=None, scale=None):
+    """Backward through sma_attn_bwd_strided; grads = (dq, dk, dv) views to fill, or None for new
+    contiguous tensors.  Returns (dq, dk, dv, delta)."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    if grads is None:
+        grads = tuple(torch.full((B, H, N, D), float("nan"), dtype=q.dtype, device=q.device) for _ in range(3))
+    dq, dk, dv = grads
+    delta = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device)
+    msb, msh = _mask_strides(packed, B, H)
+    ts = [SmaTensor.of(t) for t in (dout, q, k, v, out, dq, dk, dv)]
+    st = lib.sma_attn_bwd_strided(ts[0], ts[1], ts[2], ts[3], ts[4], lse.data_ptr(), packed.data_ptr(), msb, msh,
+                                  ts[5], ts[6], ts[7], delta.data_ptr(), B, H, N, D, scale, dt, _stream())
     assert st == SMA_OK, lib.sma_strerror(st)
     return dq, dk, dv, delta

@@ -21,12 +21,13 @@ def test_library_exports_every_declared_symbol(capi):
     header = open(os.path.join(ROOT, "include", "sma.h")).read()
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     declared = set(re.findall(r"\b(sma_[a-z_0-9]+)\s*\(", header))
-    assert {"sma_version", "sma_strerror", "sma_pack_mask", "sma_attn_fwd", "sma_attn_bwd"} <= declared
+    assert {"sma_version", "sma_strerror", "sma_pack_mask", "sma_attn_fwd", "sma_attn_bwd",
+            "sma_attn_fwd_strided", "sma_attn_bwd_strided"} <= declared
     for name in declared:
         assert hasattr(capi, name), f"{name} is declared in sma.h but not exported"
     assert capi.sma_version() >= 100
     assert capi.sma_strerror(0) == b"ok"
-    for code in range(-7, 0):
+    for code in range(-8, 0):
         assert capi.sma_strerror(code) not in (b"ok", b"unknown error code")
     assert capi.sma_strerror(-99) == b"unknown error code"
 
@@ -51,6 +52,25 @@ def test_argument_validation_needs_no_gpu(capi):
     assert call(q=ctypes.c_void_p(0x1002)) == _capi.SMA_ERR_ALIGNMENT
     assert call(B=0) == _capi.SMA_OK and call(N=0) == _capi.SMA_OK          # empty problem: nothing to do
     assert call(B=1 << 20, H=1 << 12, N=64) == _capi.SMA_ERR_BAD_SHAPE      # index range
+
+    # strided entry point: the descriptor is checked before anything is launched
+    fs = capi.sma_attn_fwd_strided
+    T = _capi.SmaTensor
+
+    def scall(q=T(0x1000, 4096, 4096, 64), msb=128, msh=128, **kw):
+        a = dict(ok_args, **kw)
+        t = T(0x1000, 4096, 4096, 64)
+        return fs(q, t, t, p, msb, msh, t, None, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
+
+    assert scall(D=128) == _capi.SMA_ERR_HEAD_DIM
+    assert scall(q=T(0x1000, 4096, 4096, 60)) == _capi.SMA_ERR_STRIDE          # not a multiple of 8 elements
+    assert scall(q=T(0x1000, 4096, -64, 64)) == _capi.SMA_ERR_STRIDE
+    assert scall(q=T(0x1000, 0, 0, 1 << 25)) == _capi.SMA_ERR_STRIDE           # (N-1) * stride_n * 2 >= 2^31
+    assert scall(q=T(None, 4096, 4096, 64)) == _capi.SMA_ERR_NULL_POINTER
+    assert scall(q=T(0x1008, 4096, 4096, 64)) == _capi.SMA_ERR_ALIGNMENT
+    assert scall(msh=-1) == _capi.SMA_ERR_STRIDE
+    assert scall(q=None) == _capi.SMA_ERR_NULL_POINTER
+    assert scall(B=0) == _capi.SMA_OK
 
     g = capi.sma_pack_mask
     assert g(None, p, 1, 1, 8, None) == _capi.SMA_ERR_NULL_POINTER
