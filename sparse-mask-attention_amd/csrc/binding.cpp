@@ -11,8 +11,13 @@
 //
 // Differences, all on the safe side: `lse` may be None (the reference's own inference wrapper
 // passes None, python/sparse_attention.py:170-171); every tensor argument is checked (device,
-// dtype, shape, contiguity, head_dim == 64) instead of only `q`; launches go to the current HIP
+// dtype, shape, layout, head_dim == 64) instead of only `q`; launches go to the current HIP
 // stream of q's device under a device guard; a failed launch raises RuntimeError.
+// q, k, v, out and the gradients need not be contiguous: any view whose last dimension is
+// contiguous and whose other strides are multiples of 8 elements is passed on with its strides
+// (the reference reserves such strides, csrc/sparse_attention.h:30-33, and ignores them), and
+// mask_packed may be [1|B, 1|H, N, ceil(N/32)]: a size of 1 shares the mask between batch
+// entries / heads.
 // This file is host-only C++ (compiled by g++); all GPU code lives behind include/sma.h.
 #include <torch/extension.h>
 #include <c10/core/DeviceGuard.h>
@@ -25,6 +30,36 @@ namespace {
 void check_status(int st, const char *what)
 {
     TORCH_CHECK(st == SMA_OK, what, " failed: ", sma_strerror(st), " (code ", st, ")");
+}
+
+// Descriptor of a [B,H,N,64] tensor for the strided C entry points.  Extents of size 1 get stride 0
+// (PyTorch leaves their strides arbitrary).
+sma_tensor rows_of(const torch::Tensor &t, const char *name)
+{
+    TORCH_CHECK(t.stride(3) == 1 || t.size(3) == 1, name, ": the last dimension must be contiguous");
+    sma_tensor d;
+    d.data = t.data_ptr();
+    d.stride_b = t.size(0) == 1 ? 0 : t.stride(0);
+    d.stride_h = t.size(1) == 1 ? 0 : t.stride(1);
+    d.stride_n = t.size(2) == 1 ? 0 : t.stride(2);
+    TORCH_CHECK(((d.stride_b | d.stride_h | d.stride_n) & 7) == 0 && d.stride_b >= 0 && d.stride_h >= 0 &&
+                    d.stride_n >= 0,
+                name, ": strides must be non-negative multiples of 8 elements (call .contiguous())");
+    return d;
+}
+
+// Checks mask_packed ([1|B, 1|H, N, nw] int32, contiguous) and returns its word strides (0 = shared).
+void mask_strides(const torch::Tensor &mp, const torch::Tensor &q, int64_t *sb, int64_t *sh)
+{
+    const int64_t B = q.size(0), H = q.size(1), N = q.size(2), nw = (N + 31) / 32;
+    TORCH_CHECK(mp.device() == q.device(), "mask_packed must be on q's device");
+    TORCH_CHECK(mp.scalar_type() == at::kInt, "mask_packed must be int32");
+    TORCH_CHECK(mp.dim() == 4 && (mp.size(0) == B || mp.size(0) == 1) && (mp.size(1) == H || mp.size(1) == 1) &&
+                    mp.size(2) == N && mp.size(3) == nw,
+                "mask_packed must be [B or 1, H or 1, N, ceil(N/32)]");
+    TORCH_CHECK(mp.is_contiguous(), "mask_packed must be contiguous");
+    *sb = mp.size(0) == 1 ? 0 : mp.size(1) * N * nw;
+    *sh = mp.size(1) == 1 ? 0 : N * nw;
 }
 
 void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,
@@ -41,16 +76,10 @@ void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor
         TORCH_CHECK(t->device() == q.device(), "q, k, v, out must be on the same device");
         TORCH_CHECK(t->scalar_type() == dt, "q, k, v, out must have the same dtype");
         TORCH_CHECK(t->sizes() == q.sizes(), "q, k, v, out must have the same shape");
-        TORCH_CHECK(t->is_contiguous(), "q, k, v, out must be contiguous");
     }
-    TORCH_CHECK(q.is_contiguous(), "q must be contiguous");
-    const int64_t nw = (N + 31) / 32;
-    TORCH_CHECK(mask_packed.device() == q.device(), "mask_packed must be on q's device");
-    TORCH_CHECK(mask_packed.scalar_type() == at::kInt, "mask_packed must be int32");
-    TORCH_CHECK(mask_packed.dim() == 4 && mask_packed.size(0) == B && mask_packed.size(1) == H &&
-                    mask_packed.size(2) == N && mask_packed.size(3) == nw,
-                "mask_packed must be [B, H, N, ceil(N/32)]");
-    TORCH_CHECK(mask_packed.is_contiguous(), "mask_packed must be contiguous");
+    const sma_tensor tq = rows_of(q, "q"), tk = rows_of(k, "k"), tv = rows_of(v, "v"), to = rows_of(out, "out");
+    int64_t msb = 0, msh = 0;
+    mask_strides(mask_packed, q, &msb, &msh);
     float *lse_ptr = nullptr;
     if (is_training) {
         TORCH_CHECK(lse.has_value() && lse->defined(), "is_training=True needs an lse tensor");
@@ -64,12 +93,11 @@ void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor
 
     const c10::DeviceGuard guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
-    const int st = sma_attn_fwd(q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                reinterpret_cast<const uint32_t *>(mask_packed.data_ptr<int32_t>()),
-                                out.data_ptr(), lse_ptr, (int)B, (int)H, (int)N, (int)D,
-                                (float)scale, dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16,
-                                stream);
-    check_status(st, "sma_attn_fwd");
+    const int st = sma_attn_fwd_strided(&tq, &tk, &tv,
+                                        reinterpret_cast<const uint32_t *>(mask_packed.data_ptr<int32_t>()),
+                                        msb, msh, &to, lse_ptr, (int)B, (int)H, (int)N, (int)D, (float)scale,
+                                        dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
+    check_status(st, "sma_attn_fwd_strided");
 }
 
 // backward(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, scale) -> None, the call the
@@ -86,19 +114,18 @@ void backward(const torch::Tensor &dout, const torch::Tensor &q, const torch::Te
     TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "Unsupported dtype, need BF16 or FP16");
     const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
     TORCH_CHECK(D == 64, "head_dim must be 64, got ", D);
-    for (const torch::Tensor *t : {&dout, &q, &k, &v, &out, static_cast<const torch::Tensor *>(&dq),
-                                   static_cast<const torch::Tensor *>(&dk),
-                                   static_cast<const torch::Tensor *>(&dv)}) {
+    const torch::Tensor *all[8] = {&dout, &q, &k, &v, &out, &dq, &dk, &dv};
+    const char *names[8] = {"dout", "q", "k", "v", "out", "dq", "dk", "dv"};
+    sma_tensor d[8];
+    for (int i = 0; i < 8; ++i) {
+        const torch::Tensor *t = all[i];
         TORCH_CHECK(t->device() == q.device(), "dout, q, k, v, out, dq, dk, dv must be on the same device");
         TORCH_CHECK(t->scalar_type() == dt, "dout, q, k, v, out, dq, dk, dv must have the same dtype");
         TORCH_CHECK(t->sizes() == q.sizes(), "dout, q, k, v, out, dq, dk, dv must have the same shape");
-        TORCH_CHECK(t->is_contiguous(), "dout, q, k, v, out, dq, dk, dv must be contiguous");
+        d[i] = rows_of(*t, names[i]);
     }
-    const int64_t nw = (N + 31) / 32;
-    TORCH_CHECK(mask_packed.device() == q.device() && mask_packed.scalar_type() == at::kInt &&
-                    mask_packed.dim() == 4 && mask_packed.size(0) == B && mask_packed.size(1) == H &&
-                    mask_packed.size(2) == N && mask_packed.size(3) == nw && mask_packed.is_contiguous(),
-                "mask_packed must be a contiguous int32 [B, H, N, ceil(N/32)] tensor on q's device");
+    int64_t msb = 0, msh = 0;
+    mask_strides(mask_packed, q, &msb, &msh);
     TORCH_CHECK(lse.device() == q.device() && lse.scalar_type() == at::kFloat && lse.dim() == 3 &&
                     lse.size(0) == B && lse.size(1) == H && lse.size(2) == N && lse.is_contiguous(),
                 "lse must be a contiguous float32 [B, H, N] tensor on q's device");
@@ -107,13 +134,12 @@ void backward(const torch::Tensor &dout, const torch::Tensor &q, const torch::Te
     const c10::DeviceGuard guard(q.device());
     torch::Tensor delta = torch::empty({B, H, N}, lse.options());      // workspace of the C entry point
     hipStream_t stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
-    const int st = sma_attn_bwd(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
-                                lse.data_ptr<float>(),
-                                reinterpret_cast<const uint32_t *>(mask_packed.data_ptr<int32_t>()),
-                                dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr<float>(),
-                                (int)B, (int)H, (int)N, (int)D, (float)scale,
-                                dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
-    check_status(st, "sma_attn_bwd");
+    const int st = sma_attn_bwd_strided(&d[0], &d[1], &d[2], &d[3], &d[4], lse.data_ptr<float>(),
+                                        reinterpret_cast<const uint32_t *>(mask_packed.data_ptr<int32_t>()),
+                                        msb, msh, &d[5], &d[6], &d[7], delta.data_ptr<float>(), (int)B, (int)H,
+                                        (int)N, (int)D, (float)scale,
+                                        dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
+    check_status(st, "sma_attn_bwd_strided");
 }
 
 torch::Tensor pack_mask(const torch::Tensor &mask)
@@ -122,6 +148,7 @@ torch::Tensor pack_mask(const torch::Tensor &mask)
     TORCH_CHECK(mask.dim() == 4, "mask must be 4D [B, H, N, N]");
     TORCH_CHECK(mask.scalar_type() == at::kBool, "mask must be bool");
     TORCH_CHECK(mask.size(2) == mask.size(3), "mask must be [B, H, N, N]");
+    // a mask shared between batch entries / heads is given as [1 or B, 1 or H, N, N] and packed as it is
     const torch::Tensor m = mask.contiguous();
     const int64_t B = m.size(0), H = m.size(1), N = m.size(2);
     TORCH_CHECK(B <= INT32_MAX && H <= INT32_MAX && N <= INT32_MAX, "extent too large");

@@ -20,6 +20,13 @@ What differs from the reference, on purpose:
   tensors live on the CPU (:148-149, :65-74), this module raises ``RuntimeError``: a silent
   fallback would hide a broken build.  ``sparse_attention_ref`` stays available for callers who
   want the PyTorch formulation explicitly.
+* ``q, k, v`` need not be contiguous: views whose last dimension is contiguous and whose other
+  strides are multiples of 8 elements (a ``[B, N, H, D]`` buffer viewed as ``[B, H, N, D]``, slices
+  of a fused qkv projection) go to the kernels as they are, where the reference would read them as
+  if they were contiguous; anything else is copied with ``.contiguous()`` first.
+* ``mask`` may be ``[1, 1, N, N]``, ``[B, 1, N, N]`` or ``[1, H, N, N]``: it is packed once at that
+  size and shared between batch entries / heads by the kernels (the reference needs the expanded
+  ``[B, H, N, N]`` tensor).
 * ``.backward()`` works.  The reference calls a ``sparse_attn_cuda.backward`` that was never
   written (:91-94); here that function exists (two HIP kernels, dQ and dK/dV, from the saved
   log-sum-exp and the packed mask).  ``backward_recompute`` states the same gradients with PyTorch
@@ -46,6 +53,14 @@ except ImportError as exc:  # the API stays importable; any compute call reports
     sparse_attn_cuda = None
     HAS_CUDA_EXT = False
     _EXT_ERROR = exc
+
+
+def _rows(t: torch.Tensor) -> torch.Tensor:
+    """t itself if the kernels can address it (contiguous last dimension, the strides of the other
+    dimensions multiples of 8 elements, 16-byte aligned storage), else a contiguous copy."""
+    ok = (t.stride(-1) == 1 or t.size(-1) == 1) and t.data_ptr() % 16 == 0 and all(
+        st % 8 == 0 for st, n in zip(t.stride()[:-1], t.shape[:-1]) if n > 1)
+    return t if ok else t.contiguous()
 
 
 def _require_ext(t: torch.Tensor) -> None:
@@ -82,7 +97,7 @@ class SparseAttentionFunction(Function):
     def forward(ctx, q, k, v, mask_packed, mask_bool, scale, seq_len):
         _require_ext(q)
         B, H, N, _ = q.shape
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        q, k, v = _rows(q), _rows(k), _rows(v)
         out = torch.empty_like(q)
         lse = torch.empty(B, H, N, device=q.device, dtype=torch.float32)
         sparse_attn_cuda.forward(q, k, v, mask_packed, out, lse, scale, True)
@@ -95,7 +110,7 @@ class SparseAttentionFunction(Function):
         q, k, v, out, lse, mask_packed = ctx.saved_tensors
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         # the call the reference makes at python/sparse_attention.py:91-94
-        sparse_attn_cuda.backward(dout.to(q.dtype).contiguous(), q, k, v, out, lse, mask_packed,
+        sparse_attn_cuda.backward(_rows(dout.to(q.dtype)), q, k, v, out, lse, mask_packed,
                                   dq, dk, dv, ctx.scale)
         return dq, dk, dv, None, None, None, None
 
@@ -124,20 +139,26 @@ def backward_recompute(q, k, v, out, lse, mask_bool, dout, scale):
 
 def _check_inputs(q, k, v, mask, mask_packed=None):
     assert q.shape == k.shape == v.shape, "q/k/v must have the same shape"
+    B, H, N, _ = q.shape
     if mask_packed is not None:
-        B, H, N, _ = q.shape
-        assert mask_packed.dtype == torch.int32 and tuple(mask_packed.shape) == (B, H, N, (N + 31) // 32), \
-            "mask_packed must be the int32 [B, H, N, ceil(N/32)] result of pack_mask"
+        mp = tuple(mask_packed.shape)
+        assert mask_packed.dtype == torch.int32 and len(mp) == 4 and mp[0] in (1, B) and mp[1] in (1, H) \
+            and mp[2:] == (N, (N + 31) // 32), \
+            "mask_packed must be the int32 [B or 1, H or 1, N, ceil(N/32)] result of pack_mask"
         assert mask_packed.device == q.device, "all tensors must be on the same device"
         return
     assert q.device == k.device == v.device == mask.device, "all tensors must be on the same device"
     assert mask.dtype == torch.bool, "mask must be a bool tensor"
+    ms = tuple(mask.shape)
+    assert len(ms) == 4 and ms[0] in (1, B) and ms[1] in (1, H) and ms[2:] == (N, N), \
+        "mask must be [B or 1, H or 1, N, N]"
 
 
 def sparse_attention(q, k, v, mask, mask_packed=None):
     """Masked attention with autograd support.
 
-    q, k, v: ``[B, H, N, D]`` (D = 64) bf16 / fp16 / fp32;  mask: bool ``[B, H, N, N]``, True = keep.
+    q, k, v: ``[B, H, N, D]`` (D = 64) bf16 / fp16 / fp32;  mask: bool ``[B, H, N, N]``, True = keep
+    (a leading extent of 1 shares the mask between batch entries / heads).
     Returns a tensor of q's shape and original dtype.
 
     ``mask_packed`` (optional, not in the reference): the result of ``pack_mask(mask)`` kept from an
@@ -174,7 +195,7 @@ def sparse_attention_func(q, k, v, mask, mask_packed=None):
         q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
 
     with torch.no_grad():
-        q, k, v = q.contiguous(), k.contiguous(), v.contiguous()
+        q, k, v = _rows(q), _rows(k), _rows(v)
         if mask_packed is None:
             mask_packed = pack_mask(mask)
         out = torch.empty_like(q)
@@ -190,7 +211,8 @@ def sparse_attention_func(q, k, v, mask, mask_packed=None):
 # ----------------------------------------------------------------------------------------------
 
 def pack_mask(mask: torch.Tensor) -> torch.Tensor:
-    """bool ``[B, H, N, N]`` -> bit-packed int32 ``[B, H, N, ceil(N/32)]`` (bit j of word w = column 32w+j)."""
+    """bool ``[B, H, N, N]`` -> bit-packed int32 ``[B, H, N, ceil(N/32)]`` (bit j of word w = column 32w+j).
+    A mask shared between batch entries / heads is passed (and packed) as ``[1 or B, 1 or H, N, N]``."""
     _require_ext(mask)
     return sparse_attn_cuda.pack_mask(mask)
 

@@ -196,3 +196,51 @@ def test_forward_can_be_captured_in_a_graph_and_replayed(sa, dev):
         eager = sa.sparse_attention_func(qd, kd, vd, md)
         torch.cuda.synchronize()
         assert torch.equal(out_g, eager), f"replay {rep}"
+
+
+@pytest.mark.parametrize("mshape", ["11", "B1", "BH"])
+def test_views_of_a_fused_projection_and_shared_masks_through_autograd(sa, dev, mshape):
+    """q, k, v as slices of one [B, N, 3, H, D] projection output (no copies are made), the mask
+    shared between heads and/or batch entries; output and gradients against the oracle on the
+    expanded mask.  The gradient arrives through a transpose, so dout is a strided view as well."""
+    B, H, N = 2, 3, 136
+    g = torch.Generator().manual_seed(21)
+    qkv = torch.randn(B, N, 3, H, 64, generator=g).to(torch.float16)
+    Bm, Hm = (1 if mshape[0] == "1" else B), (1 if mshape[1] == "1" else H)
+    mask = torch.rand(Bm, Hm, N, N, generator=g) < 0.3
+    mask[..., 5, :] = False
+    leaf = qkv.to(dev).requires_grad_(True)
+    q, k, v = (leaf[:, :, i].permute(0, 2, 1, 3) for i in range(3))          # [B, H, N, D] views
+    assert sa._rows(q) is q and not q.is_contiguous()
+    out = sa.sparse_attention(q, k, v, mask.to(dev))
+    w = torch.randn(B, N, H, 64, generator=g).to(torch.float16)
+    (out.permute(0, 2, 1, 3) * w.to(dev)).sum().backward()
+
+    ref_leaf = qkv.float().requires_grad_(True)
+    rq, rk, rv = (ref_leaf[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    ref = O.sparse_attention_ref(rq, rk, rv, mask.expand(B, H, N, N))
+    (ref.permute(0, 2, 1, 3) * w.float()).sum().backward()
+    assert torch.allclose(out.float().cpu(), ref.detach(), atol=1e-2, rtol=1e-2)
+    assert (out[:, :, 5] == 0).all()
+    bound = 1e-4 + 1e-2 * ref_leaf.grad.abs().max() + 2e-2 * ref_leaf.grad.abs()
+    assert ((leaf.grad.float().cpu() - ref_leaf.grad).abs() <= bound).all()
+    # the packed mask has the mask's own leading extents and can be reused
+    packed = sa.pack_mask(mask.to(dev))
+    assert packed.shape == (Bm, Hm, N, (N + 31) // 32)
+    again = sa.sparse_attention_func(q.detach(), k.detach(), v.detach(), None, mask_packed=packed)
+    assert torch.equal(again, out.detach())
+
+
+def test_layouts_the_kernels_cannot_address_are_copied(sa, dev):
+    """Odd strides (rows of 72 elements are fine, rows of 68 are not) and a transposed last dimension."""
+    q, k, v, mask = _inputs(1, 2, 64, torch.float16, 8)
+    md = mask.to(dev)
+    want = sa.sparse_attention_func(q.to(dev), k.to(dev), v.to(dev), md)
+    for pad in (72, 68):
+        store = torch.zeros(1, 2, 64, pad, dtype=torch.float16, device=dev)
+        store[..., :64] = q.to(dev)
+        view = store[..., :64]
+        assert (sa._rows(view) is view) == (pad == 72)
+        assert torch.equal(sa.sparse_attention_func(view, k.to(dev), v.to(dev), md), want)
+    qt = q.to(dev).transpose(2, 3).contiguous().transpose(2, 3)
+    assert torch.equal(sa.sparse_attention_func(qt, k.to(dev), v.to(dev), md), want)
