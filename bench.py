@@ -10,6 +10,7 @@ Prints ONE JSON line.  Besides the whole-step figure it carries
   roofline      the fused attention kernel alone (the dominant kernel) against the dense FP16 MFMA
                 peak, from stream-event timing of back-to-back launches on the launch stream;
   roofline_pack the packer alone against the HBM peak;
+  roofline_bwd  the backward (its two kernels, one call) against the MFMA peak, 2.5 x the forward's FLOP;
   cpu_baseline  the oracle's PyTorch formulation of the same workload on the host cores.
 """
 import argparse
@@ -46,18 +47,23 @@ def event_time_ms(fn, warmup, repeat, torch):
     return start.elapsed_time(end) / repeat
 
 
-def measured_traffic(kernel, workload):
-    """HBM bytes per launch from the committed rocprofv3 counter summary of this kernel and workload
-    (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a plain copy of known
-    size); None when no summary for this workload is there.  Counters cannot be read from inside
-    this process, so the figure is the recorded one, not a live one."""
+def measured_traffic(workload, *kernels):
+    """HBM bytes per launch (summed over `kernels`) from the committed rocprofv3 counter summaries
+    of this workload (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a
+    plain copy of known size); None when a summary for this workload is not there.  Counters cannot
+    be read from inside this process, so the figure is the recorded one, not a live one."""
     import re
-    path = os.path.join(ROOT, "profiles", f"{kernel}_{workload}.txt")
-    try:
-        m = re.search(r"traffic per launch ([0-9.]+) MB", open(path).read())
-    except OSError:
-        return None
-    return int(float(m.group(1)) * 1e6) if m else None
+    total = 0
+    for kernel in kernels:
+        path = os.path.join(ROOT, "profiles", f"{kernel}_{workload}.txt")
+        try:
+            m = re.search(r"traffic per launch ([0-9.]+) MB", open(path).read())
+        except OSError:
+            return None
+        if not m:
+            return None
+        total += int(float(m.group(1)) * 1e6)
+    return total
 
 
 def main():
@@ -127,6 +133,14 @@ def main():
     pack_ms = event_time_ms(lambda: lib.sma_pack_mask(md.data_ptr(), packed.data_ptr(), w.B, w.H, w.N, stream),
                             10, reps, torch)
     api_ms = event_time_ms(lambda: sa.sparse_attention_func(qd, kd, vd, md), 10, reps, torch)
+    # the backward (dQ kernel, then dK/dV kernel) on the forward's saved out and lse
+    lse = torch.empty(w.B, w.H, w.N, dtype=torch.float32, device=dev)
+    ext.forward(qd, kd, vd, packed, out, lse, scale, True)
+    dout = torch.randn(qd.shape, generator=torch.Generator().manual_seed(43)).to(qd.dtype).to(dev)
+    dq, dk, dv = (torch.empty_like(qd) for _ in range(3))
+    bwd_ms = event_time_ms(lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale),
+                           5, reps, torch)
+    bwd_tflops = w.bwd_dense_flops / (bwd_ms * 1e-3) / 1e12
 
     # FLOP the kernel really executes: 32-row x 64-key blocks of the mask that hold a set bit
     # (a wavefront skips the others), 4*32*64*D each, so that skipping is not mistaken for MFMA speed
@@ -160,15 +174,20 @@ def main():
         "attn_kernel_executed_tflops": round(executed_flops / (attn_ms * 1e-3) / 1e12, 2),
         "attn_live_block_fraction": round(executed_flops / w.dense_flops, 4) if w.N % 64 == 0 else None,
         "pack_kernel_ms": round(pack_ms, 5),
+        "backward_ms": round(bwd_ms, 5),
         "api_sparse_attention_func_ms": round(api_ms, 5),
         "roofline": {"kernel": "attn_fwd_kernel", "bound": "mfma", "achieved": round(attn_tflops, 2),
                      "peak": harness.MI355X_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
                      "frac": round(attn_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4),
-                     "traffic": measured_traffic("attn_fwd_kernel", w.name), "algorithmic_bytes": w.attn_bytes},
+                     "traffic": measured_traffic(w.name, "attn_fwd_kernel"), "algorithmic_bytes": w.attn_bytes},
         "roofline_pack": {"kernel": "pack_flat_kernel" if w.N % 32 == 0 else ("pack_row8_kernel" if w.N % 8 == 0 else "pack_rows_kernel"),
                           "bound": "hbm", "achieved": round(pack_gbps, 1), "peak": harness.MI355X_HBM_GBPS,
                           "unit": "GB/s", "frac": round(pack_gbps / harness.MI355X_HBM_GBPS, 4),
-                          "traffic": measured_traffic("pack_mask_kernel", w.name), "algorithmic_bytes": w.pack_bytes},
+                          "traffic": measured_traffic(w.name, "pack_mask_kernel"), "algorithmic_bytes": w.pack_bytes},
+        "roofline_bwd": {"kernel": "attn_bwd_dq_kernel + attn_bwd_dkv_kernel", "bound": "mfma",
+                         "achieved": round(bwd_tflops, 2), "peak": harness.MI355X_MFMA_F16_TFLOPS,
+                         "unit": "TFLOP/s", "frac": round(bwd_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4),
+                         "traffic": measured_traffic(w.name, "attn_bwd_dq_kernel", "attn_bwd_dkv_kernel"), "algorithmic_bytes": w.bwd_bytes},
     }
 
     if not args.no_cpu_baseline:

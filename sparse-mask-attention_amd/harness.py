@@ -50,6 +50,23 @@ class Workload:
         return 4 * self.B * self.H * self.N * self.D * 2 + 4 * self.B * self.H * self.N * self.n_words
 
     @property
+    def bwd_dense_flops(self) -> int:
+        """Dense-equivalent FLOP of the backward, by the usual convention 2.5 x the forward: the five
+        N x N x D products dV, dP, dQ, dK and the recomputed S (what the kernels execute is seven,
+        S and dP are formed in both)."""
+        return 10 * self.B * self.H * self.N * self.N * self.D
+
+    @property
+    def bwd_bytes(self) -> int:
+        """Algorithmic bytes of one backward (both launches): the dQ kernel reads q, k, v, dout, out,
+        the mask and lse and writes dq and delta; the dK/dV kernel reads q, k, v, dout, the mask, lse
+        and delta and writes dk and dv."""
+        mat = self.B * self.H * self.N * self.D * 2
+        mask = 4 * self.B * self.H * self.N * self.n_words
+        vec = 4 * self.B * self.H * self.N
+        return (6 * mat + mask + 2 * vec) + (6 * mat + mask + 2 * vec)
+
+    @property
     def pack_bytes(self) -> int:
         """Algorithmic bytes of one pack_mask launch: one byte in per entry + the words out."""
         return self.B * self.H * self.N * self.N + 4 * self.B * self.H * self.N * self.n_words
