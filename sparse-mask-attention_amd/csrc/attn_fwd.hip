@@ -42,28 +42,43 @@
 namespace sma {
 namespace {
 
-constexpr int HD = 64;             // head dim
+constexpr int HD = 64;             // columns of one LDS tile: the head dim, or one half of a head dim of 128
 constexpr int BM = 128;            // query rows per work-group
 constexpr int BN = 64;             // keys per tile
 constexpr int NTHREADS = 256;
 constexpr int TILE_BYTES = BN * HD * 2;          // 8 KiB, rows of 128 B
-constexpr int NSTAGE = 3;
 constexpr float WINDOW_LOG2 = 8.0f;
 
-// LDS map (bytes)
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;                 // K then V
-constexpr int OFF_MASK = NSTAGE * STAGE_BYTES;              // 3 slots x 4 waves x 64 words
-constexpr int OFF_LUT = OFF_MASK + 3 * 1024;                // 16 x 16 B
-constexpr int LDS_BYTES = OFF_LUT + 256;
+// Head dim 64 * NH.  A head dim of 128 is handled as two column halves of 64: K and V tiles are kept
+// in LDS as two 64-column tiles each (same row length, swizzles and read patterns as for 64), the
+// QK^T chain runs over both halves of K and q, and P multiplies each half of V into its own pair
+// of accumulators.  Its stage is twice as large, so the ring has two stages (copies one tile
+// ahead) and two work-groups share a CU.
+template <int NH> struct Cfg {
+    static constexpr int NSTAGE = NH == 1 ? 3 : 2;
+    static constexpr int WAVES_PER_SIMD = NH == 1 ? 3 : 2;
+    static constexpr int COPIES = 1 + 4 * NH;                       // async copies per wave and tile
+    // LDS map (bytes)
+    static constexpr int STAGE_BYTES = 2 * NH * TILE_BYTES;         // K halves, then V halves
+    static constexpr int OFF_V = NH * TILE_BYTES;                   // V inside a stage
+    static constexpr int OFF_MASK = NSTAGE * STAGE_BYTES;           // NSTAGE slots x 4 waves x 64 words
+    static constexpr int OFF_LUT = OFF_MASK + NSTAGE * 1024;        // 16 x 16 B
+    static constexpr int LDS_BYTES = OFF_LUT + 256;
+};
+
+template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
 
 // PACKED_ROWS: the rows of q, k, v and out follow each other without gaps (row stride 64), as in
 // contiguous tensors; the strides between heads and batch entries stay free.  A row stride known
 // at compile time measured 0.25 us less fixed cost per launch than the same value read at run time.
-template <bool BF16, bool POSTMUL, bool PACKED_ROWS>
-__global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
+template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int NH>
+__global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_kernel(const AttnArgs a)
 {
     using E = Elem<BF16>;
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
+    using C = Cfg<NH>;
+    constexpr int NSTAGE = C::NSTAGE, STAGE_BYTES = C::STAGE_BYTES, OFF_MASK = C::OFF_MASK, OFF_LUT = C::OFF_LUT;
+    constexpr int D = HD * NH;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[C::LDS_BYTES];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem;
 
     const int tid = threadIdx.x;
@@ -93,22 +108,22 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     const uint16_t *kb = slab(a.k, bi, hi);
     const uint16_t *vb = slab(a.v, bi, hi);
     const uint32_t *mb = slab(a.mask, bi, hi);
-    const uint32_t q_sn = PACKED_ROWS ? HD : a.q.sn, k_sn = PACKED_ROWS ? HD : a.k.sn;     // row strides, elements
-    const uint32_t v_sn = PACKED_ROWS ? HD : a.v.sn, o_sn = PACKED_ROWS ? HD : a.out.sn;
+    const uint32_t q_sn = PACKED_ROWS ? D : a.q.sn, k_sn = PACKED_ROWS ? D : a.k.sn;       // row strides, elements
+    const uint32_t v_sn = PACKED_ROWS ? D : a.v.sn, o_sn = PACKED_ROWS ? D : a.out.sn;
     const uint32_t q_rb = 2u * q_sn, k_rb = 2u * k_sn, v_rb = 2u * v_sn;                   // row pitch, bytes
 
-    // ---- mask words: wave-private async copies, slot = tile % 3, lane i -> (row i/2, word i%2) ----
+    // ---- mask words: wave-private async copies, slot = tile % NSTAGE, lane i -> (row i/2, word i%2) ----
     const int mrow = qt * BM + wave * 32 + (lane >> 1);
     const uint32_t m_voff = (uint32_t)(((size_t)(mrow < N ? mrow : N - 1) * nw + (lane & 1)) * 4);
     const uint32_t mask_dst = lds0 + wave * 256;
-    auto issue_mask = [&](int x, auto slot_c) {
+    auto issue_mask = [&](int x, auto slot_c) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
         uint32_t voff = m_voff;
         if (2 * x + 1 >= nw) voff -= (lane & 1) * 4;           // odd word count: re-read the last word
         async_copy_b32_at<OFF_MASK + SLOT * 1024>(mask_dst, mb + 2 * x, voff);
     };
     const uint32_t maddr = lds0 + OFF_MASK + wave * 256 + l32 * 8;
-    auto mask_words = [&](int x, int slot) -> u32x2 {
+    auto mask_words = [&](int x, int slot) __attribute__((always_inline)) -> u32x2 {
         u32x2 w = lds_read_b64(maddr + slot * 1024);
         const bool last = (x == T - 1);
         w.x &= last ? a.last_mask0 : 0xffffffffu;
@@ -131,7 +146,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         kv_voff[1][j] = __umul24(row, v_rb) + ((pos ^ fr) << 4);
     }
     const uint32_t kv_dst = lds0 + wave * 2048;
-    auto issue_kv = [&](int t, auto stage_c) {
+    auto issue_kv = [&](int t, auto stage_c) __attribute__((always_inline)) {
         constexpr int SO = decltype(stage_c)::value * STAGE_BYTES;
         const int key0 = t * BN;
         uint32_t ko[2] = {kv_voff[0][0], kv_voff[0][1]}, vo[2] = {kv_voff[1][0], kv_voff[1][1]};
@@ -148,10 +163,18 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         const uint16_t *ksrc = kb + (size_t)key0 * k_sn, *vsrc = vb + (size_t)key0 * v_sn;
         async_copy_b128_at<SO>(kv_dst, ksrc, ko[0]);
         async_copy_b128_at<SO + 1024>(kv_dst, ksrc, ko[1]);
-        async_copy_b128_at<SO + TILE_BYTES>(kv_dst, vsrc, vo[0]);
-        async_copy_b128_at<SO + TILE_BYTES + 1024>(kv_dst, vsrc, vo[1]);
+        if constexpr (NH == 2) {              // second column half: 128 bytes further along each row
+            async_copy_b128_at<SO + TILE_BYTES>(kv_dst, ksrc + HD, ko[0]);
+            async_copy_b128_at<SO + TILE_BYTES + 1024>(kv_dst, ksrc + HD, ko[1]);
+        }
+        async_copy_b128_at<SO + C::OFF_V>(kv_dst, vsrc, vo[0]);
+        async_copy_b128_at<SO + C::OFF_V + 1024>(kv_dst, vsrc, vo[1]);
+        if constexpr (NH == 2) {
+            async_copy_b128_at<SO + C::OFF_V + TILE_BYTES>(kv_dst, vsrc + HD, vo[0]);
+            async_copy_b128_at<SO + C::OFF_V + TILE_BYTES + 1024>(kv_dst, vsrc + HD, vo[1]);
+        }
     };
-    auto zero_tail_rows = [&](int t, int stage) {   // after the copies of the last tile have landed
+    auto zero_tail_rows = [&](int t, int stage) __attribute__((always_inline)) {   // after the copies of the last tile have landed
         const int key0 = t * BN;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
@@ -159,13 +182,13 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
             if (key0 + row >= N) {
                 const uint32_t p = lds0 + stage * STAGE_BYTES + wave * 2048 + j * 1024 + lane * 16;
                 const u32x4 z = {0u, 0u, 0u, 0u};
-                *(LDS_PTR(u32x4))(uintptr_t)p = z;
-                *(LDS_PTR(u32x4))(uintptr_t)(p + TILE_BYTES) = z;
+#pragma unroll
+                for (int part = 0; part < 2 * NH; ++part) *(LDS_PTR(u32x4))(uintptr_t)(p + part * TILE_BYTES) = z;
             }
         }
     };
 
-    // ---- per-lane LDS read addresses (stage 0); everything else is an immediate offset ----
+    // ---- per-lane LDS read addresses (stage 0, first column half); everything else is an immediate offset ----
     // K operand (blk, s): row 32*blk + l32, chunk 2s + hh           -> kaddr[s] + 4096*blk
     // V operand (dblk, blk, u, x), read by ds_read_b64_tr_b16: the lane supplies
     //   row 32blk + 16u + 8x + 4hh + (i >> 2), columns 32dblk + 16G + 4(i & 3) .. +3
@@ -185,7 +208,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
 #pragma unroll
             for (int dblk = 0; dblk < 2; ++dblk) {
                 const int chunk = 4 * dblk + 2 * G + ((i16 & 3) >> 1);
-                vaddr[dblk][x] = lds0 + TILE_BYTES + row * 128 + ((chunk ^ fr) << 4) + ((i16 & 1) << 3);
+                vaddr[dblk][x] = lds0 + C::OFF_V + row * 128 + ((chunk ^ fr) << 4) + ((i16 & 1) << 3);
             }
         }
     }
@@ -193,20 +216,23 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     const uint32_t nib_shift = 4u - 4u * hh;
 
     // ================================ prologue: one memory round trip ================================
-    // Requested at once, oldest first: q (this wave's 32 rows, staged through the still unused third
-    // K/V stage, K-swizzled), then the mask words and K/V of tiles 0 and 1.
+    // Requested at once, oldest first: q (this wave's 32 rows, staged through the last K/V stage,
+    // which the prologue leaves unused, K-swizzled), then the mask words and K/V of the first
+    // NSTAGE - 1 tiles.
     const int qrow = qt * BM + wave * 32 + l32;
     {
         const int qbase = qt * BM + wave * 32 < N ? qt * BM + wave * 32 : N - 1;   // wave-uniform
         const uint16_t *qsrc = qb + (size_t)qbase * q_sn;
         const int last = N - 1 - qbase;                      // rows beyond N re-read row N-1
-        const uint32_t dst = lds0 + 2 * STAGE_BYTES + wave * 4096;
+        const uint32_t dst = lds0 + (NSTAGE - 1) * STAGE_BYTES + wave * 4096;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int row = 8 * j + (lane >> 3);
             const int pos = lane & 7;
             const int lrow = row < last ? row : last;
-            async_copy_b128(dst + j * 1024, qsrc, __umul24(lrow, q_rb) + ((pos ^ ((row >> 1) & 7)) << 4));
+            const uint32_t voff = __umul24(lrow, q_rb) + ((pos ^ ((row >> 1) & 7)) << 4);
+            async_copy_b128(dst + j * 1024, qsrc, voff);
+            if constexpr (NH == 2) async_copy_b128(dst + 16384 + j * 1024, qsrc + HD, voff);
         }
     }
     using std::integral_constant;
@@ -215,17 +241,20 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     // small LDS table for the mask: entry n (16 B) holds four floats, float j = (bit j of n) ? 0 : -inf
     if (tid < 64)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
-    const bool even_progress = (int)blockIdx.x >= a.tail_start;
+    const bool even_progress = NH == 1 && (int)blockIdx.x >= a.tail_start;
     if (even_progress && T >= 4) __builtin_amdgcn_s_setprio(3);
-    if (T > 1) { issue_mask(1, integral_constant<int, 1>{}); issue_kv(1, integral_constant<int, 1>{}); }
-
-    if (T > 1) WAIT_VMCNT(10); else WAIT_VMCNT(5);       // q has landed
+    if constexpr (NSTAGE == 3) {
+        if (T > 1) { issue_mask(1, integral_constant<int, 1>{}); issue_kv(1, integral_constant<int, 1>{}); }
+        if (T > 1) wait_vmcnt<2 * C::COPIES>(); else wait_vmcnt<C::COPIES>();       // q has landed
+    } else {
+        wait_vmcnt<C::COPIES>();
+    }
     // ---- Q^T as MFMA B operands, scaled by scale*log2(e)/post_mul:
     //      lane holds query row l32, d = 16*s + 8*hh .. +7
-    u32x4 qf[4];
+    u32x4 qf[4 * NH];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
-        u32x4 t = lds_read_b128(kaddr[s] + 2 * STAGE_BYTES + wave * 4096);
+    for (int s = 0; s < 4 * NH; ++s) {
+        u32x4 t = lds_read_b128(kaddr[s & 3] + (NSTAGE - 1) * STAGE_BYTES + (s >> 2) * 16384 + wave * 4096);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const float lo = E::up1((uint16_t)(t[i] & 0xffffu)) * a.q_scale;
@@ -236,9 +265,11 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     }
 
     // ---- running state: one query row per lane; both lane halves hold the same ref ----
-    f32x16 oacc[2];
+    f32x16 oacc[2 * NH];                // [2 * half + dblk]: 32 columns each
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { oacc[0][i] = 0.f; oacc[1][i] = 0.f; }
+    for (int b = 0; b < 2 * NH; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[b][i] = 0.f;
     float ref = 0.f;                    // reference point r, in accumulator units (log2 / pm)
     float rmax = -__builtin_inff();     // largest score seen so far minus r; -inf = none yet
     float l_run = 0.f;                  // this lane's share of sum exp2(pm * (score - r))
@@ -247,7 +278,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
     u32x4 ones = {E::ONES, E::ONES, E::ONES, E::ONES};
     asm volatile("" : "+v"(ones));      // keep the constant operand resident in registers
 
-    auto set_ref = [&](float r_wanted) -> float {      // returns the value actually represented
+    auto set_ref = [&](float r_wanted) __attribute__((always_inline)) -> float {      // returns the value actually represented
         float rest = -r_wanted, sum = 0.f;
         uint16_t term[4];
 #pragma unroll
@@ -266,7 +297,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
 
     // One key tile for this wavefront.  `so` (LDS offset of the stage) is a compile-time constant
     // in every call, so all LDS addresses below are a register plus an immediate.
-    auto compute_tile = [&](const u32x2 w2, const uint32_t so) {
+    auto compute_tile = [&](const u32x2 w2, const uint32_t so) __attribute__((always_inline)) {
         if (__builtin_amdgcn_ballot_w64((w2.x | w2.y) != 0u) == 0ull) return;
         // ---- S^T: sacc[blk][4g+j] = log2 weight / pm of (key 32blk + 8g + 4hh + j, query l32) ----
         f32x16 sacc[2];
@@ -285,9 +316,10 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
             sacc[1] = E::mfma(ones, refb, sacc[1]);
         }
 #pragma unroll
-        for (int s = 0; s < 4; ++s) {
-            sacc[0] = E::mfma(lds_read_b128(kaddr[s] + so), qf[s], sacc[0]);
-            sacc[1] = E::mfma(lds_read_b128(kaddr[s] + so + 4096), qf[s], sacc[1]);
+        for (int s = 0; s < 4 * NH; ++s) {
+            const uint32_t ka = kaddr[s & 3] + so + (s >> 2) * TILE_BYTES;
+            sacc[0] = E::mfma(lds_read_b128(ka), qf[s], sacc[0]);
+            sacc[1] = E::mfma(lds_read_b128(ka + 4096), qf[s], sacc[1]);
         }
         // ---- row max over this tile; move the reference only when the window is left ----
         float mx = -__builtin_inff();
@@ -311,7 +343,8 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
             l_run *= alpha;
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
-                oacc[0][i] *= alpha; oacc[1][i] *= alpha;
+#pragma unroll
+                for (int b = 0; b < 2 * NH; ++b) oacc[b][i] *= alpha;
                 sacc[0][i] += delta; sacc[1][i] += delta;
             }
             rmax = top + delta;
@@ -335,7 +368,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
                     lsum = E::add2(pk, lsum);
                 }
         l_run += lsum;
-        // ---- O^T += V^T * P^T : oacc[dblk][4g+j] = out(query l32, d = 32dblk + 8g + 4hh + j) ----
+        // ---- O^T += V^T * P^T : oacc[b][4g+j] = out(query l32, d = 32b + 8g + 4hh + j) ----
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
@@ -343,26 +376,27 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
                 const u32x4 pv = {pb[blk][u][0], pb[blk][u][1], pb[blk][u][2], pb[blk][u][3]};
                 const uint32_t off = so + 4096 * blk + 2048 * u;
 #pragma unroll
-                for (int dblk = 0; dblk < 2; ++dblk) {
-                    const u32x2 lo = lds_read_tr16_b64(vaddr[dblk][0] + off);
-                    const u32x2 hi = lds_read_tr16_b64(vaddr[dblk][1] + off);
+                for (int b = 0; b < 2 * NH; ++b) {
+                    const uint32_t voff = off + (b >> 1) * TILE_BYTES;
+                    const u32x2 lo = lds_read_tr16_b64(vaddr[b & 1][0] + voff);
+                    const u32x2 hi = lds_read_tr16_b64(vaddr[b & 1][1] + voff);
                     const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
-                    oacc[dblk] = E::mfma(va, pv, oacc[dblk]);
+                    oacc[b] = E::mfma(va, pv, oacc[b]);
                 }
             }
     };
 
     // ================================ main loop ================================
-    // Tile t uses stage and mask slot t % 3; the loop is unrolled by 3 so that these are
+    // Tile t uses stage and mask slot t % NSTAGE; the loop is unrolled by NSTAGE so that these are
     // constants.  In iteration t:
-    //   wait for the copies of tile t  ->  barrier  ->  request the copies of tile t + 2 (mask
-    //   words, then K/V)  ->  compute, unless this wave's 32 x 64 block of mask bits is empty.
+    //   wait for the copies of tile t  ->  barrier  ->  request the copies of tile t + NSTAGE - 1
+    //   (mask words, then K/V)  ->  compute, unless this wave's 32 x 64 block of mask bits is empty.
     // Every tile is copied: exchanging per-tile "is any of the 128 rows live" flags between the
     // waves (tried: through LDS two tiles ahead, and as a bit map built up front from the mask
     // rows) cost more than the copies it saved, on block-structured masks too.
-    auto iteration = [&](const int t, auto slot_c) {
+    auto iteration = [&](const int t, auto slot_c) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
-        constexpr int SLOT2 = (SLOT + 2) % 3;
+        constexpr int SLOT2 = (SLOT + NSTAGE - 1) % NSTAGE;       // the stage freed by the barrier below
         if (even_progress) {
             // The hardware serves the oldest wave first, so of three co-resident work-groups one
             // finishes early and the last runs alone, at a worse rate than three together.  When
@@ -371,43 +405,49 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
             else if (t == T / 2) __builtin_amdgcn_s_setprio(1);
             else if (t == (3 * T) / 4) __builtin_amdgcn_s_setprio(0);
         }
-        // copies complete in issue order; only those of the next tile (5) may stay in flight
-        if (t + 1 < T) WAIT_VMCNT(5); else WAIT_VMCNT(0);
+        // copies complete in issue order; only those of the tiles requested after tile t may stay in flight
+        if (NSTAGE == 3 && t + 1 < T) wait_vmcnt<C::COPIES>(); else wait_vmcnt<0>();
         if (ragged && t == T - 1) zero_tail_rows(t, SLOT);
         __syncthreads();          // tile t landed for every wave; the stage of tile t - 1 is free
         const u32x2 w2 = mask_words(t, SLOT);
-        if (t + 2 < T) { issue_mask(t + 2, integral_constant<int, SLOT2>{}); issue_kv(t + 2, integral_constant<int, SLOT2>{}); }
+        if (t + NSTAGE - 1 < T) {
+            issue_mask(t + NSTAGE - 1, integral_constant<int, SLOT2>{});
+            issue_kv(t + NSTAGE - 1, integral_constant<int, SLOT2>{});
+        }
         compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
     };
-    for (int t = 0; t < T; t += 3) {
+    for (int t = 0; t < T; t += NSTAGE) {
         iteration(t, integral_constant<int, 0>{});
         if (t + 1 < T) iteration(t + 1, integral_constant<int, 1>{});
-        if (t + 2 < T) iteration(t + 2, integral_constant<int, 2>{});
+        if constexpr (NSTAGE == 3) {
+            if (t + 2 < T) iteration(t + 2, integral_constant<int, 2>{});
+        }
     }
-    WAIT_VMCNT(0);                // no copy may outlive the work-group's LDS allocation
+    wait_vmcnt<0>();              // no copy may outlive the work-group's LDS allocation
 
     // ---- epilogue ----
     // out = O / l.  The accumulator layout gives a lane 8-byte pieces of one row; written as they
     // are, a store instruction would touch 32 different 128-byte rows.  Each wave therefore
-    // transposes its 32 x 64 block through 4 KiB of LDS (K/V stage 0, free after a barrier; chunks
-    // XOR-swizzled as for K) and stores whole rows: 8 lanes x 16 B per row, 8 rows per instruction.
+    // transposes its 32 x 64 block (one per column half) through 4 KiB of LDS (K/V stage 0, free
+    // after a barrier; chunks XOR-swizzled as for K) and stores whole 128-byte pieces of rows: 8 lanes
+    // x 16 B per row, 8 rows per instruction.
     const float l_tot = xhalf_sum(l_run);
     const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
     __syncthreads();              // every wave is done reading the K/V stages
     {
-        const uint32_t obase = lds0 + wave * 4096;
+        const uint32_t obase = lds0 + wave * 4096;           // + 16 KiB for the second column half
         const uint32_t wrow = obase + l32 * 128 + hh * 8;
         const int fo = (l32 >> 1) & 7;
 #pragma unroll
-        for (int dblk = 0; dblk < 2; ++dblk)
+        for (int b = 0; b < 2 * NH; ++b)
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const uint32_t lo = (uint32_t)E::cvt1(oacc[dblk][4 * g + 0] * inv) |
-                                    ((uint32_t)E::cvt1(oacc[dblk][4 * g + 1] * inv) << 16);
-                const uint32_t hi = (uint32_t)E::cvt1(oacc[dblk][4 * g + 2] * inv) |
-                                    ((uint32_t)E::cvt1(oacc[dblk][4 * g + 3] * inv) << 16);
+                const uint32_t lo = (uint32_t)E::cvt1(oacc[b][4 * g + 0] * inv) |
+                                    ((uint32_t)E::cvt1(oacc[b][4 * g + 1] * inv) << 16);
+                const uint32_t hi = (uint32_t)E::cvt1(oacc[b][4 * g + 2] * inv) |
+                                    ((uint32_t)E::cvt1(oacc[b][4 * g + 3] * inv) << 16);
                 const u32x2 o = {lo, hi};
-                *(LDS_PTR(u32x2))(uintptr_t)(wrow + (((4 * dblk + g) ^ fo) << 4)) = o;
+                *(LDS_PTR(u32x2))(uintptr_t)(wrow + (b >> 1) * 16384 + (((4 * (b & 1) + g) ^ fo) << 4)) = o;
             }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
@@ -415,12 +455,15 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_fwd_kernel(const AttnArgs a)
         const int row0 = qt * BM + wave * 32;
         uint16_t *ob = slab(a.out, bi, hi) + (size_t)row0 * o_sn;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int row = 8 * j + (lane >> 3), pos = lane & 7;
-            const u32x4 v = lds_read_b128(obase + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
-            // non-temporal: the output is not read again here and should not displace K, V and the mask
-            if (row0 + row < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(ob + (size_t)row * o_sn + pos * 8));
-        }
+        for (int half = 0; half < NH; ++half)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int row = 8 * j + (lane >> 3), pos = lane & 7;
+                const u32x4 v = lds_read_b128(obase + half * 16384 + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
+                // non-temporal: the output is not read again here and should not displace K, V and the mask
+                if (row0 + row < N)
+                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(ob + (size_t)row * o_sn + half * HD + pos * 8));
+            }
     }
     if (qrow < N) {
         if (a.lse != nullptr && hh == 0) {
@@ -460,17 +503,27 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     a.tail_start = (groups > 2 * cus && groups <= 3 * cus) ? 0 : (int)groups;
     const dim3 grid((unsigned)groups), block(NTHREADS);
     const bool postmul = a.post_mul != 1.0f;
-    const bool packed = a.q.sn == HD && a.k.sn == HD && a.v.sn == HD && a.out.sn == HD;
+    const int D = a.D;
+    const bool packed = (int)a.q.sn == D && (int)a.k.sn == D && (int)a.v.sn == D && (int)a.out.sn == D;
+    if (D != HD) a.tail_start = (int)groups;                  // two work-groups per CU: nobody yields
     void (*kernel)(const AttnArgs) = nullptr;
-    switch ((bf16 ? 4 : 0) | (postmul ? 2 : 0) | (packed ? 1 : 0)) {
-    case 0: kernel = attn_fwd_kernel<false, false, false>; break;
-    case 1: kernel = attn_fwd_kernel<false, false, true>; break;
-    case 2: kernel = attn_fwd_kernel<false, true, false>; break;
-    case 3: kernel = attn_fwd_kernel<false, true, true>; break;
-    case 4: kernel = attn_fwd_kernel<true, false, false>; break;
-    case 5: kernel = attn_fwd_kernel<true, false, true>; break;
-    case 6: kernel = attn_fwd_kernel<true, true, false>; break;
-    default: kernel = attn_fwd_kernel<true, true, true>; break;
+    switch ((D == 2 * HD ? 8 : 0) | (bf16 ? 4 : 0) | (postmul ? 2 : 0) | (packed ? 1 : 0)) {
+    case 0: kernel = attn_fwd_kernel<false, false, false, 1>; break;
+    case 1: kernel = attn_fwd_kernel<false, false, true, 1>; break;
+    case 2: kernel = attn_fwd_kernel<false, true, false, 1>; break;
+    case 3: kernel = attn_fwd_kernel<false, true, true, 1>; break;
+    case 4: kernel = attn_fwd_kernel<true, false, false, 1>; break;
+    case 5: kernel = attn_fwd_kernel<true, false, true, 1>; break;
+    case 6: kernel = attn_fwd_kernel<true, true, false, 1>; break;
+    case 7: kernel = attn_fwd_kernel<true, true, true, 1>; break;
+    case 8: kernel = attn_fwd_kernel<false, false, false, 2>; break;
+    case 9: kernel = attn_fwd_kernel<false, false, true, 2>; break;
+    case 10: kernel = attn_fwd_kernel<false, true, false, 2>; break;
+    case 11: kernel = attn_fwd_kernel<false, true, true, 2>; break;
+    case 12: kernel = attn_fwd_kernel<true, false, false, 2>; break;
+    case 13: kernel = attn_fwd_kernel<true, false, true, 2>; break;
+    case 14: kernel = attn_fwd_kernel<true, true, false, 2>; break;
+    default: kernel = attn_fwd_kernel<true, true, true, 2>; break;
     }
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, a);
     return hipGetLastError();

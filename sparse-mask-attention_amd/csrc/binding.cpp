@@ -11,7 +11,7 @@
 //
 // Differences, all on the safe side: `lse` may be None (the reference's own inference wrapper
 // passes None, python/sparse_attention.py:170-171); every tensor argument is checked (device,
-// dtype, shape, layout, head_dim == 64) instead of only `q`; launches go to the current HIP
+// dtype, shape, layout, head_dim 64 or 128 (backward: 64)) instead of only `q`; launches go to the current HIP
 // stream of q's device under a device guard; a failed launch raises RuntimeError.
 // q, k, v, out and the gradients need not be contiguous: any view whose last dimension is
 // contiguous and whose other strides are multiples of 8 elements is passed on with its strides
@@ -32,7 +32,7 @@ void check_status(int st, const char *what)
     TORCH_CHECK(st == SMA_OK, what, " failed: ", sma_strerror(st), " (code ", st, ")");
 }
 
-// Descriptor of a [B,H,N,64] tensor for the strided C entry points.  Extents of size 1 get stride 0
+// Descriptor of a [B,H,N,D] tensor for the strided C entry points.  Extents of size 1 get stride 0
 // (PyTorch leaves their strides arbitrary).
 sma_tensor rows_of(const torch::Tensor &t, const char *name)
 {
@@ -71,7 +71,7 @@ void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor
     const auto dt = q.scalar_type();
     TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "Unsupported dtype, need BF16 or FP16");
     const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
-    TORCH_CHECK(D == 64, "head_dim must be 64, got ", D);
+    TORCH_CHECK(D == 64 || D == 128, "head_dim must be 64 or 128, got ", D);
     for (const torch::Tensor *t : {&k, &v, static_cast<const torch::Tensor *>(&out)}) {
         TORCH_CHECK(t->device() == q.device(), "q, k, v, out must be on the same device");
         TORCH_CHECK(t->scalar_type() == dt, "q, k, v, out must have the same dtype");

@@ -13,14 +13,14 @@ inline sma_tensor dense(const void *p, int H, int N, int D)
     return sma_tensor{const_cast<void *>(p), (int64_t)H * N * D, (int64_t)N * D, (int64_t)D};
 }
 
-// Checks one strided [B,H,N,64] tensor and converts it; SMA_OK or an error code.
-int to_rows(const sma_tensor *t, int N, sma::Rows *r)
+// Checks one strided [B,H,N,D] tensor and converts it; SMA_OK or an error code.
+int to_rows(const sma_tensor *t, int N, int D, sma::Rows *r)
 {
     if (t == nullptr || t->data == nullptr) return SMA_ERR_NULL_POINTER;
     if (misaligned(t->data, 16)) return SMA_ERR_ALIGNMENT;
     if (t->stride_b < 0 || t->stride_h < 0 || t->stride_n < 0) return SMA_ERR_STRIDE;
     if ((t->stride_b | t->stride_h | t->stride_n) & 7) return SMA_ERR_STRIDE;
-    if ((long long)(N - 1) * t->stride_n * 2 + 128 >= (1ll << 31)) return SMA_ERR_STRIDE;
+    if ((long long)(N - 1) * t->stride_n * 2 + 2 * D >= (1ll << 31)) return SMA_ERR_STRIDE;
     if (t->stride_b >= (1ll << 35) || t->stride_h >= (1ll << 35) || t->stride_n >= (1ll << 23)) return SMA_ERR_STRIDE;
     r->p = static_cast<uint16_t *>(t->data);
     r->sb8 = (uint32_t)(t->stride_b >> 3);
@@ -41,7 +41,7 @@ const char *sma_strerror(int code)
     case SMA_OK:               return "ok";
     case SMA_ERR_NULL_POINTER: return "a required pointer is NULL";
     case SMA_ERR_BAD_SHAPE:    return "bad shape: negative extent or index range exceeded";
-    case SMA_ERR_HEAD_DIM:     return "unsupported head_dim (only 64)";
+    case SMA_ERR_HEAD_DIM:     return "unsupported head_dim (forward: 64 or 128; backward: 64)";
     case SMA_ERR_DTYPE:        return "unsupported dtype (need fp16 or bf16)";
     case SMA_ERR_SCALE:        return "scale must be finite";
     case SMA_ERR_LAUNCH:       return "HIP kernel launch failed";
@@ -113,7 +113,7 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
     const sma_tensor *in[8] = {dout, q, k, v, out, dq, dk, dv};
     sma::Rows *to[8] = {&a.dout, &a.q, &a.k, &a.v, &a.out, &a.dq, &a.dk, &a.dv};
     for (int i = 0; i < 8; ++i) {
-        const int st = to_rows(in[i], N, to[i]);
+        const int st = to_rows(in[i], N, D, to[i]);
         if (st != SMA_OK) return st;
     }
     a.lse = lse;
@@ -136,7 +136,7 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
                          int dtype, void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
-    if (D != 64) return SMA_ERR_HEAD_DIM;
+    if (D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
     if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
     if (!isfinite(scale)) return SMA_ERR_SCALE;
     const long long BH = (long long)B * H;
@@ -151,7 +151,7 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
     const sma_tensor *in[4] = {q, k, v, out};
     sma::Rows *to[4] = {&a.q, &a.k, &a.v, &a.out};
     for (int i = 0; i < 4; ++i) {
-        const int st = to_rows(in[i], N, to[i]);
+        const int st = to_rows(in[i], N, D, to[i]);
         if (st != SMA_OK) return st;
     }
     a.mask = sma::PackedMask{mask_packed, mask_stride_b, mask_stride_h};
@@ -159,6 +159,7 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
     a.BH = (int)BH;
     a.H = H;
     a.N = N;
+    a.D = D;
     a.qtiles = (int)qtiles;
     split_scale(scale, &a.q_scale, &a.post_mul);
     last_tile_masks(N, &a.last_mask0, &a.last_mask1);

@@ -42,7 +42,8 @@ def test_argument_validation_needs_no_gpu(capi):
         return f(q, k, v, mp, out, lse, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
 
     assert call(D=32) == _capi.SMA_ERR_HEAD_DIM
-    assert call(D=128) == _capi.SMA_ERR_HEAD_DIM
+    assert call(D=96) == _capi.SMA_ERR_HEAD_DIM
+    assert call(D=256) == _capi.SMA_ERR_HEAD_DIM
     assert call(dtype=2) == _capi.SMA_ERR_DTYPE
     assert call(B=-1) == _capi.SMA_ERR_BAD_SHAPE
     assert call(scale=float("nan")) == _capi.SMA_ERR_SCALE
@@ -62,7 +63,7 @@ def test_argument_validation_needs_no_gpu(capi):
         t = T(0x1000, 4096, 4096, 64)
         return fs(q, t, t, p, msb, msh, t, None, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
 
-    assert scall(D=128) == _capi.SMA_ERR_HEAD_DIM
+    assert scall(D=96) == _capi.SMA_ERR_HEAD_DIM
     assert scall(q=T(0x1000, 4096, 4096, 60)) == _capi.SMA_ERR_STRIDE          # not a multiple of 8 elements
     assert scall(q=T(0x1000, 4096, -64, 64)) == _capi.SMA_ERR_STRIDE
     assert scall(q=T(0x1000, 0, 0, 1 << 25)) == _capi.SMA_ERR_STRIDE           # (N-1) * stride_n * 2 >= 2^31
