@@ -22,7 +22,7 @@ extern "C" {
 #define SMA_OK                 0
 #define SMA_ERR_NULL_POINTER  -1   /* a required pointer is NULL */
 #define SMA_ERR_BAD_SHAPE     -2   /* a negative extent, or an extent beyond the 32-bit index range */
-#define SMA_ERR_HEAD_DIM      -3   /* head_dim other than 64 or 128 (forward) / 64 (backward) */
+#define SMA_ERR_HEAD_DIM      -3   /* head_dim other than 64 or 128 */
 #define SMA_ERR_DTYPE         -4   /* dtype other than SMA_DTYPE_F16 / SMA_DTYPE_BF16 */
 #define SMA_ERR_SCALE         -5   /* scale is NaN or infinite */
 #define SMA_ERR_LAUNCH        -6   /* the HIP runtime refused the launch (hipGetLastError) */
@@ -74,7 +74,7 @@ int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *ma
 
 /* Masked attention backward:  given dout = dLoss/dout, the gradients with respect to q, k and v.
  *
- *   dout, q, k, v, out  [B,H,N,D] fp16 or bf16 (dtype), D must be 64; out and lse are the results
+ *   dout, q, k, v, out  [B,H,N,D] fp16 or bf16 (dtype), D 64 or 128; out and lse are the results
  *                       of sma_attn_fwd on the same q, k, v, mask_packed and scale
  *   lse                 float [B,H,N] as written by sma_attn_fwd (-inf for rows that keep no key)
  *   mask_packed         uint32 [B,H,N,ceil(N/32)]
@@ -83,7 +83,8 @@ int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *ma
  *   delta_ws            float [B,H,N] workspace owned by the caller; holds sum_d dout*out per query
  *                       row on return (the library never allocates)
  *
- * Two launches on `stream` (dq, then dk and dv); no atomics, results are bit-reproducible.
+ * Two launches on `stream` (dq, then dk and dv; three for D = 128: dq, dk, dv); no atomics, results are
+ * bit-reproducible.
  *
  * Replaces: void sparse_attention_bwd_bf16(const SparseAttentionParams&, const void* dout,
  *           void* dq, void* dk, void* dv, cudaStream_t), declared csrc/sparse_attention.h:57-64 and

@@ -25,23 +25,35 @@
 // stages, one tile ahead; the 16-byte chunks of a row are XOR-swizzled with bitrev3((row >> 1) & 7),
 // which keeps both the row reads (ds_read_b128) and the transposing reads (ds_read_b64_tr_b16) of
 // the same tile free of bank conflicts.
+//
+// Head dim 128 (NH = 2) is handled as two column halves of 64: every streamed matrix is kept in LDS
+// as two 64-column tiles, the products that contract over the head dim (S, dP) run over both
+// halves, the others (dQ, dK, dV) fill one pair of accumulators per half.  The dK/dV kernel would
+// need 128 accumulator registers for that; it is therefore launched twice, once for dK and once
+// for dV (S is formed in both).
 #include "attn_common.h"
 
 namespace sma {
 namespace {
 
-constexpr int HD = 64;
+constexpr int HD = 64;             // columns of one LDS tile: the head dim, or one half of a head dim of 128
 constexpr int BM = 128;            // rows (queries or keys) per work-group
 constexpr int BN = 64;             // rows per streamed tile
 constexpr int NTHREADS = 256;
 constexpr int TILE_BYTES = BN * HD * 2;
-constexpr int STAGE_BYTES = 2 * TILE_BYTES;
 constexpr int NSTAGE = 2;
 constexpr int AUX_BYTES = 2048;                             // small per-tile data of a stage
-constexpr int OFF_AUX = NSTAGE * STAGE_BYTES;
-constexpr int OFF_LUT = OFF_AUX + NSTAGE * AUX_BYTES;
-constexpr int LDS_BYTES = OFF_LUT + 256;
 constexpr float LOG2E = 1.4426950408889634f;
+
+// LDS map (bytes) for head dim 64 * NH: a stage holds the NH column halves of the first streamed
+// matrix, then those of the second.
+template <int NH> struct Cfg {
+    static constexpr int STAGE_BYTES = 2 * NH * TILE_BYTES;
+    static constexpr int OFF_B = NH * TILE_BYTES;           // second matrix inside a stage
+    static constexpr int OFF_AUX = NSTAGE * STAGE_BYTES;
+    static constexpr int OFF_LUT = OFF_AUX + NSTAGE * AUX_BYTES;
+    static constexpr int LDS_BYTES = OFF_LUT + 256;
+};
 
 __device__ __forceinline__ int bitrev3(int f) { return ((f & 1) << 2) | (f & 2) | (f >> 2); }
 
@@ -66,6 +78,7 @@ __device__ __forceinline__ TileCopy make_tile_copy(int wave, int lane)
 }
 // Copy the tile whose first row is row r0 of the N-row matrix `mat` (row stride sn elements, below
 // 2^23); rows >= N re-read row N-1 (they are zeroed after landing).
+template <int NH>
 __device__ __forceinline__ void issue_tile(uint32_t dst, const uint16_t *mat, uint32_t sn, int r0,
                                            int N, const TileCopy &c, int wave)
 {
@@ -74,17 +87,21 @@ __device__ __forceinline__ void issue_tile(uint32_t dst, const uint16_t *mat, ui
 #pragma unroll
     for (int j = 0; j < 2; ++j) {
         const int r = c.row[j] < last ? c.row[j] : last;
-        async_copy_b128(dst + wave * 2048 + j * 1024, src, __umul24(r, 2u * sn) + c.chunk[j]);
+        const uint32_t voff = __umul24(r, 2u * sn) + c.chunk[j];
+        async_copy_b128(dst + wave * 2048 + j * 1024, src, voff);
+        if constexpr (NH == 2) async_copy_b128(dst + TILE_BYTES + wave * 2048 + j * 1024, src + HD, voff);
     }
 }
-__device__ __forceinline__ void zero_tile_tail(uint32_t dst, int r0, int N, const TileCopy &c,
+// Zero the rows >= N of the `parts` consecutive 64-column tiles that start at dst.
+__device__ __forceinline__ void zero_tile_tail(uint32_t dst, int parts, int r0, int N, const TileCopy &c,
                                                int wave, int lane)
 {
 #pragma unroll
     for (int j = 0; j < 2; ++j)
         if (r0 + c.row[j] >= N) {
             const u32x4 z = {0u, 0u, 0u, 0u};
-            *(LDS_PTR(u32x4))(uintptr_t)(dst + wave * 2048 + j * 1024 + lane * 16) = z;
+            for (int part = 0; part < parts; ++part)
+                *(LDS_PTR(u32x4))(uintptr_t)(dst + part * TILE_BYTES + wave * 2048 + j * 1024 + lane * 16) = z;
         }
 }
 
@@ -135,12 +152,14 @@ __device__ __forceinline__ u32x4 load_frag(const uint16_t *mat, int sn, int row,
 }
 
 // Transposed store of a 32 x 64 accumulator block (acc[dblk][4g+j] = value(row l32, column
-// 32dblk + 8g + 4hh + j)) times `mult`, through 4 KiB of wave-private LDS, as whole 128-byte rows
-// (dst_row0: the block's first row; sn: row stride in elements).
+// 32dblk + 8g + 4hh + j), acc = {acc0, acc1}) times `mult`, through 4 KiB of wave-private LDS, as
+// whole 128-byte pieces of rows (dst_row0: first row, first of the 64 columns; sn: row stride in
+// elements).
 template <bool BF16>
-__device__ __forceinline__ void store_block(const f32x16 (&acc)[2], float mult, uint32_t lds_wave,
+__device__ __forceinline__ void store_block(const f32x16 &acc0, const f32x16 &acc1, float mult, uint32_t lds_wave,
                                             uint16_t *dst_row0, int sn, int row0, int N, int lane)
 {
+    const f32x16 acc[2] = {acc0, acc1};
     using E = Elem<BF16>;
     const int l32 = lane & 31, hh = lane >> 5;
     const uint32_t wrow = lds_wave + l32 * 128 + hh * 8;
@@ -170,11 +189,13 @@ __device__ __forceinline__ void store_block(const f32x16 (&acc)[2], float mult, 
 // ------------------------------------------------------------------------------------------------
 // dQ (and delta)
 // ------------------------------------------------------------------------------------------------
-template <bool BF16>
-__global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdArgs a)
+template <bool BF16, int NH>
+__global__ __launch_bounds__(NTHREADS, NH == 1 ? 3 : 2) void attn_bwd_dq_kernel(const AttnBwdArgs a)
 {
     using E = Elem<BF16>;
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
+    using C = Cfg<NH>;
+    constexpr int STAGE_BYTES = C::STAGE_BYTES, OFF_AUX = C::OFF_AUX, OFF_LUT = C::OFF_LUT;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[C::LDS_BYTES];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem;
 
     const int tid = threadIdx.x;
@@ -197,10 +218,10 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdA
     // ---- this lane's query row: q^T and dO^T fragments (B operands), delta, lse ----
     const int qrow = qt * BM + wave * 32 + l32;
     const int qr = qrow < N ? qrow : N - 1;
-    u32x4 qf[4], dof[4];
+    u32x4 qf[4 * NH], dof[4 * NH];
     float delta = 0.f;
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int s = 0; s < 4 * NH; ++s) {
         const int col = 16 * s + 8 * hh;
         u32x4 tq = load_frag(qb, a.q.sn, qr, col);
         const u32x4 td = load_frag(dob, a.dout.sn, qr, col);
@@ -231,16 +252,18 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdA
         uint32_t voff = m_voff;
         if (2 * t + 1 >= nw) voff -= (lane & 1) * 4;          // odd word count: re-read the last word
         async_copy_b32(lds0 + OFF_AUX + st * AUX_BYTES + wave * 256, mb + 2 * t, voff);
-        issue_tile(lds0 + st * STAGE_BYTES, kb, a.k.sn, t * BN, N, tc, wave);
-        issue_tile(lds0 + st * STAGE_BYTES + TILE_BYTES, vb, a.v.sn, t * BN, N, tc, wave);
+        issue_tile<NH>(lds0 + st * STAGE_BYTES, kb, a.k.sn, t * BN, N, tc, wave);
+        issue_tile<NH>(lds0 + st * STAGE_BYTES + C::OFF_B, vb, a.v.sn, t * BN, N, tc, wave);
     };
     issue(0, 0);
     if (tid < 64)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
 
-    f32x16 oacc[2];
+    f32x16 oacc[2 * NH];                // [2 * half + dblk]: 32 columns of dQ each
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { oacc[0][i] = 0.f; oacc[1][i] = 0.f; }
+    for (int b = 0; b < 2 * NH; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) oacc[b][i] = 0.f;
     const uint32_t lut_addr = lds0 + OFF_LUT;
     const uint32_t nib_shift = 4u - 4u * hh;
 
@@ -248,10 +271,7 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdA
         const int st = t & 1;
         const uint32_t so = lds0 + st * STAGE_BYTES;
         WAIT_VMCNT(0);
-        if (ragged && t == T - 1) {
-            zero_tile_tail(so, t * BN, N, tc, wave, lane);
-            zero_tile_tail(so + TILE_BYTES, t * BN, N, tc, wave, lane);
-        }
+        if (ragged && t == T - 1) zero_tile_tail(so, 2 * NH, t * BN, N, tc, wave, lane);
         __syncthreads();          // tile t of every wave landed; the other stage is free
         if (t + 1 < T) issue(t + 1, st ^ 1);
 
@@ -276,9 +296,10 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdA
                 }
             }
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-                sacc = E::mfma(lds_read_b128(tr.rowaddr[s] + so + 4096 * blk), qf[s], sacc);
-                dacc = E::mfma(lds_read_b128(tr.rowaddr[s] + so + TILE_BYTES + 4096 * blk), dof[s], dacc);
+            for (int s = 0; s < 4 * NH; ++s) {
+                const uint32_t ra = tr.rowaddr[s & 3] + so + (s >> 2) * TILE_BYTES + 4096 * blk;
+                sacc = E::mfma(lds_read_b128(ra), qf[s], sacc);
+                dacc = E::mfma(lds_read_b128(ra + C::OFF_B), dof[s], dacc);
             }
 #pragma unroll
             for (int u = 0; u < 2; ++u)
@@ -298,30 +319,38 @@ __global__ __launch_bounds__(NTHREADS, 3) void attn_bwd_dq_kernel(const AttnBwdA
                 const u32x4 pv = {pb[blk][u][0], pb[blk][u][1], pb[blk][u][2], pb[blk][u][3]};
                 const uint32_t off = so + 4096 * blk + 2048 * u;
 #pragma unroll
-                for (int dblk = 0; dblk < 2; ++dblk) {
-                    const u32x2 lo = lds_read_tr16_b64(tr.traddr[dblk][0] + off);
-                    const u32x2 hi = lds_read_tr16_b64(tr.traddr[dblk][1] + off);
+                for (int b = 0; b < 2 * NH; ++b) {
+                    const uint32_t ko = off + (b >> 1) * TILE_BYTES;
+                    const u32x2 lo = lds_read_tr16_b64(tr.traddr[b & 1][0] + ko);
+                    const u32x2 hi = lds_read_tr16_b64(tr.traddr[b & 1][1] + ko);
                     const u32x4 va = {lo.x, lo.y, hi.x, hi.y};
-                    oacc[dblk] = E::mfma(va, pv, oacc[dblk]);
+                    oacc[b] = E::mfma(va, pv, oacc[b]);
                 }
             }
     }
     WAIT_VMCNT(0);
     __syncthreads();              // every wave is done reading the stages
     const int row0 = qt * BM + wave * 32;
-    if (row0 < N)
-        store_block<BF16>(oacc, a.scale, lds0 + wave * 4096, slab(a.dq, bi, hi) + (size_t)row0 * a.dq.sn,
-                          a.dq.sn, row0, N, lane);
+    if (row0 < N) {
+#pragma unroll
+        for (int half = 0; half < NH; ++half)
+            store_block<BF16>(oacc[2 * half], oacc[2 * half + 1], a.scale, lds0 + wave * 4096,
+                              slab(a.dq, bi, hi) + (size_t)row0 * a.dq.sn + half * HD, a.dq.sn, row0, N, lane);
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
 // dK and dV
 // ------------------------------------------------------------------------------------------------
-template <bool BF16>
+// DK / DV: which of the two gradients this instance produces (both for head dim 64; one per launch
+// for head dim 128, where both sets of accumulators do not fit the register file).
+template <bool BF16, int NH, bool DK, bool DV>
 __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwdArgs a)
 {
     using E = Elem<BF16>;
-    __shared__ __attribute__((aligned(1024))) unsigned char smem[LDS_BYTES];
+    using C = Cfg<NH>;
+    constexpr int STAGE_BYTES = C::STAGE_BYTES, OFF_AUX = C::OFF_AUX;
+    __shared__ __attribute__((aligned(1024))) unsigned char smem[C::LDS_BYTES];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem;
 
     const int tid = threadIdx.x;
@@ -349,12 +378,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     const int kr = key < N ? key : N - 1;
     const uint32_t key_ok = key < N ? 0xffffffffu : 0u;
     const int wi = (key0 >> 5) < nw ? (key0 >> 5) : nw - 1;     // this wave's mask word of a row
-    u32x4 kf[4], vf[4];
+    u32x4 kf[4 * NH], vf[DK ? 4 * NH : 1];
 #pragma unroll
-    for (int s = 0; s < 4; ++s) {
+    for (int s = 0; s < 4 * NH; ++s) {
         const int col = 16 * s + 8 * hh;
         u32x4 tk = load_frag(kb, a.k.sn, kr, col);
-        vf[s] = load_frag(vb, a.v.sn, kr, col);
+        if constexpr (DK) vf[s] = load_frag(vb, a.v.sn, kr, col);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
             const float lo = E::up1((uint16_t)(tk[i] & 0xffffu)) * a.q_scale;
@@ -374,14 +403,19 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
         async_copy_b32(aux + wave * 256, mb + wi, (uint32_t)((size_t)row * nw * 4));
         if (wave == 0) async_copy_b32(aux + 1024, lse_b, (uint32_t)(row * 4));
         if (wave == 1) async_copy_b32(aux + 1280, delta_b, (uint32_t)(row * 4));
-        issue_tile(lds0 + st * STAGE_BYTES, qb, a.q.sn, r0, N, tc, wave);
-        issue_tile(lds0 + st * STAGE_BYTES + TILE_BYTES, dob, a.dout.sn, r0, N, tc, wave);
+        issue_tile<NH>(lds0 + st * STAGE_BYTES, qb, a.q.sn, r0, N, tc, wave);
+        issue_tile<NH>(lds0 + st * STAGE_BYTES + C::OFF_B, dob, a.dout.sn, r0, N, tc, wave);
     };
     issue(0, 0);
 
-    f32x16 dkacc[2], dvacc[2];
+    f32x16 dkacc[DK ? 2 * NH : 1], dvacc[DV ? 2 * NH : 1];      // [2 * half + dblk]: 32 columns each
 #pragma unroll
-    for (int i = 0; i < 16; ++i) { dkacc[0][i] = 0.f; dkacc[1][i] = 0.f; dvacc[0][i] = 0.f; dvacc[1][i] = 0.f; }
+    for (int b = 0; b < 2 * NH; ++b)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            if constexpr (DK) dkacc[b][i] = 0.f;
+            if constexpr (DV) dvacc[b][i] = 0.f;
+        }
 
     for (int t = 0; t < T; ++t) {
         const int st = t & 1;
@@ -395,10 +429,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
             const bool dead = (t * BN + lane >= N) || (l == -__builtin_inff());
             *(LDS_PTR(float))(uintptr_t)p = dead ? __builtin_inff() : l * LOG2E;
         }
-        if (ragged && t == T - 1) {
-            zero_tile_tail(so, t * BN, N, tc, wave, lane);
-            zero_tile_tail(so + TILE_BYTES, t * BN, N, tc, wave, lane);
-        }
+        if (ragged && t == T - 1) zero_tile_tail(so, 2 * NH, t * BN, N, tc, wave, lane);
         __syncthreads();
         if (t + 1 < T) issue(t + 1, st ^ 1);
         if (!wave_valid) continue;
@@ -420,17 +451,21 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
 #pragma unroll
             for (int i = 0; i < 16; ++i) { sacc[i] = 0.f; dacc[i] = 0.f; }
 #pragma unroll
-            for (int s = 0; s < 4; ++s)
-                sacc = E::mfma(lds_read_b128(tr.rowaddr[s] + so + 4096 * blk), kf[s], sacc);
+            for (int s = 0; s < 4 * NH; ++s)
+                sacc = E::mfma(lds_read_b128(tr.rowaddr[s & 3] + so + (s >> 2) * TILE_BYTES + 4096 * blk), kf[s], sacc);
+            if constexpr (DK) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s)
-                dacc = E::mfma(lds_read_b128(tr.rowaddr[s] + so + TILE_BYTES + 4096 * blk), vf[s], dacc);
+                for (int s = 0; s < 4 * NH; ++s)
+                    dacc = E::mfma(lds_read_b128(tr.rowaddr[s & 3] + so + C::OFF_B + (s >> 2) * TILE_BYTES + 4096 * blk),
+                                   vf[s], dacc);
+            }
 
-            uint32_t pp[2][4], ps[2][4];
+            uint32_t pp[2][4] = {}, ps[2][4] = {};       // the one a single-gradient instance leaves unused is dropped
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
                 const u32x4 Lr = lds_read_b128(aux + 1024 + rsel + 32 * g);
-                const u32x4 Dr = lds_read_b128(aux + 1280 + rsel + 32 * g);
+                u32x4 Dr = {0u, 0u, 0u, 0u};
+                if constexpr (DK) Dr = lds_read_b128(aux + 1280 + rsel + 32 * g);
                 float p[4], d[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
@@ -442,10 +477,14 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
                     d[j] = p[j] * (dacc[4 * g + j] - Dj);
                 }
                 // elements 4g .. 4g+3 are pairs (2i, 2i+1) with i = 2(g & 1), 2(g & 1) + 1 of u = g >> 1
-                pp[g >> 1][2 * (g & 1)] = E::pack2_rne(p[0], p[1]);
-                pp[g >> 1][2 * (g & 1) + 1] = E::pack2_rne(p[2], p[3]);
-                ps[g >> 1][2 * (g & 1)] = E::pack2_rne(d[0], d[1]);
-                ps[g >> 1][2 * (g & 1) + 1] = E::pack2_rne(d[2], d[3]);
+                if constexpr (DV) {
+                    pp[g >> 1][2 * (g & 1)] = E::pack2_rne(p[0], p[1]);
+                    pp[g >> 1][2 * (g & 1) + 1] = E::pack2_rne(p[2], p[3]);
+                }
+                if constexpr (DK) {
+                    ps[g >> 1][2 * (g & 1)] = E::pack2_rne(d[0], d[1]);
+                    ps[g >> 1][2 * (g & 1) + 1] = E::pack2_rne(d[2], d[3]);
+                }
             }
 #pragma unroll
             for (int u = 0; u < 2; ++u) {
@@ -453,15 +492,20 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
                 const u32x4 bs = {ps[u][0], ps[u][1], ps[u][2], ps[u][3]};
                 const uint32_t off = so + 4096 * blk + 2048 * u;
 #pragma unroll
-                for (int dblk = 0; dblk < 2; ++dblk) {
-                    const u32x2 qlo = lds_read_tr16_b64(tr.traddr[dblk][0] + off);
-                    const u32x2 qhi = lds_read_tr16_b64(tr.traddr[dblk][1] + off);
-                    const u32x2 dlo = lds_read_tr16_b64(tr.traddr[dblk][0] + off + TILE_BYTES);
-                    const u32x2 dhi = lds_read_tr16_b64(tr.traddr[dblk][1] + off + TILE_BYTES);
-                    const u32x4 qa = {qlo.x, qlo.y, qhi.x, qhi.y};
-                    const u32x4 da = {dlo.x, dlo.y, dhi.x, dhi.y};
-                    dkacc[dblk] = E::mfma(qa, bs, dkacc[dblk]);      // dK^T += Q^T dS
-                    dvacc[dblk] = E::mfma(da, bp, dvacc[dblk]);      // dV^T += dO^T P
+                for (int b = 0; b < 2 * NH; ++b) {
+                    const uint32_t ho = off + (b >> 1) * TILE_BYTES;
+                    if constexpr (DK) {                              // dK^T += Q^T dS
+                        const u32x2 qlo = lds_read_tr16_b64(tr.traddr[b & 1][0] + ho);
+                        const u32x2 qhi = lds_read_tr16_b64(tr.traddr[b & 1][1] + ho);
+                        const u32x4 qa = {qlo.x, qlo.y, qhi.x, qhi.y};
+                        dkacc[b] = E::mfma(qa, bs, dkacc[b]);
+                    }
+                    if constexpr (DV) {                              // dV^T += dO^T P
+                        const u32x2 dlo = lds_read_tr16_b64(tr.traddr[b & 1][0] + ho + C::OFF_B);
+                        const u32x2 dhi = lds_read_tr16_b64(tr.traddr[b & 1][1] + ho + C::OFF_B);
+                        const u32x4 da = {dlo.x, dlo.y, dhi.x, dhi.y};
+                        dvacc[b] = E::mfma(da, bp, dvacc[b]);
+                    }
                 }
             }
         }
@@ -469,10 +513,15 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     WAIT_VMCNT(0);
     __syncthreads();
     if (wave_valid) {
-        store_block<BF16>(dkacc, a.scale, lds0 + wave * 4096, slab(a.dk, bi, hi) + (size_t)key0 * a.dk.sn,
-                          a.dk.sn, key0, N, lane);
-        store_block<BF16>(dvacc, 1.0f, lds0 + wave * 4096, slab(a.dv, bi, hi) + (size_t)key0 * a.dv.sn,
-                          a.dv.sn, key0, N, lane);
+#pragma unroll
+        for (int half = 0; half < NH; ++half) {
+            if constexpr (DK)
+                store_block<BF16>(dkacc[2 * half], dkacc[2 * half + 1], a.scale, lds0 + wave * 4096,
+                                  slab(a.dk, bi, hi) + (size_t)key0 * a.dk.sn + half * HD, a.dk.sn, key0, N, lane);
+            if constexpr (DV)
+                store_block<BF16>(dvacc[2 * half], dvacc[2 * half + 1], 1.0f, lds0 + wave * 4096,
+                                  slab(a.dv, bi, hi) + (size_t)key0 * a.dv.sn + half * HD, a.dv.sn, key0, N, lane);
+        }
     }
 }
 
@@ -487,12 +536,24 @@ hipError_t launch_attn_bwd(const AttnBwdArgs &args, bool bf16, hipStream_t strea
     if (groups == 0) return hipSuccess;
     const dim3 grid((unsigned)groups), block(NTHREADS);
     // dQ first: it also fills the delta workspace that the dK/dV kernel reads (same stream).
-    if (bf16) {
-        hipLaunchKernelGGL((attn_bwd_dq_kernel<true>), grid, block, 0, stream, a);
-        hipLaunchKernelGGL((attn_bwd_dkv_kernel<true>), grid, block, 0, stream, a);
+    if (a.D == HD) {
+        if (bf16) {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 1>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 1, true, true>), grid, block, 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 1>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 1, true, true>), grid, block, 0, stream, a);
+        }
     } else {
-        hipLaunchKernelGGL((attn_bwd_dq_kernel<false>), grid, block, 0, stream, a);
-        hipLaunchKernelGGL((attn_bwd_dkv_kernel<false>), grid, block, 0, stream, a);
+        if (bf16) {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 2>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 2, true, false>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 2, false, true>), grid, block, 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 2>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 2, true, false>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 2, false, true>), grid, block, 0, stream, a);
+        }
     }
     return hipGetLastError();
 }

@@ -41,7 +41,7 @@ const char *sma_strerror(int code)
     case SMA_OK:               return "ok";
     case SMA_ERR_NULL_POINTER: return "a required pointer is NULL";
     case SMA_ERR_BAD_SHAPE:    return "bad shape: negative extent or index range exceeded";
-    case SMA_ERR_HEAD_DIM:     return "unsupported head_dim (forward: 64 or 128; backward: 64)";
+    case SMA_ERR_HEAD_DIM:     return "unsupported head_dim (64 or 128)";
     case SMA_ERR_DTYPE:        return "unsupported dtype (need fp16 or bf16)";
     case SMA_ERR_SCALE:        return "scale must be finite";
     case SMA_ERR_LAUNCH:       return "HIP kernel launch failed";
@@ -98,7 +98,7 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
                          void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
-    if (D != 64) return SMA_ERR_HEAD_DIM;
+    if (D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
     if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
     if (!isfinite(scale)) return SMA_ERR_SCALE;
     const long long BH = (long long)B * H;
@@ -122,6 +122,7 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
     a.BH = (int)BH;
     a.H = H;
     a.N = N;
+    a.D = D;
     a.qtiles = (int)qtiles;
     a.scale = scale;
     split_scale(scale, &a.q_scale, &a.post_mul);

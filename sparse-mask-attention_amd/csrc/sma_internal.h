@@ -73,6 +73,7 @@ struct AttnBwdArgs {
     Rows dq, dk, dv;
     float *delta;                              // [BH, N] workspace: sum_d dout * out per query row
     int BH, H, N;
+    int D;                                     // head dim: 64 or 128
     int qtiles;                                // ceil(N / 128)
     FastDiv div_qtiles, div_H;                 // filled in by the launcher
     float scale;                               // as given by the caller
