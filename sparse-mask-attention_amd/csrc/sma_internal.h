@@ -7,7 +7,7 @@
 
 namespace sma {
 
-// A [B, H, N, 64] tensor of 16-bit elements (fp16 or bf16 bit patterns).  The 64 elements of a row
+// A [B, H, N, D] tensor of 16-bit elements (fp16 or bf16 bit patterns).  The D elements of a row
 // are contiguous; the other extents have strides that are multiples of 8 elements (rows stay
 // 16-byte aligned).  Byte offsets inside one (b, h) slab fit 31 bits (checked by the C-ABI layer).
 // Kept small: kernel arguments are fetched by every work-group before it can request any data.

@@ -197,3 +197,31 @@ def test_python_api_head_dim_128_autograd(dev):
     for got, want in zip(leaves, refs):
         bound = 1e-4 + 1e-2 * want.grad.abs().max() + 2e-2 * want.grad.abs()
         assert ((got.grad.float().cpu() - want.grad).abs() <= bound).all()
+
+
+@pytest.mark.parametrize("D", [32, 80, 96, 128])
+def test_python_api_other_head_dims(dev, D):
+    """Head dims without a kernel of their own are zero-padded by the Python layer; results and
+    gradients must be those of the operator at that head dim (scale 1/sqrt(D))."""
+    import importlib
+    import sys
+    importlib.import_module("python.sparse_attention")
+    sa = sys.modules["python.sparse_attention"]
+    g = torch.Generator().manual_seed(40 + D)
+    q, k, v = [torch.randn(2, 2, 120, D, generator=g).to(torch.float16) for _ in range(3)]
+    mask = torch.rand(2, 2, 120, 120, generator=g) < 0.35
+    leaves = [t.to(dev).requires_grad_(True) for t in (q, k, v)]
+    out = sa.sparse_attention(*leaves, mask.to(dev))
+    assert out.shape == (2, 2, 120, D)
+    w = torch.randn(out.shape, generator=g).to(torch.float16)
+    out.backward(w.to(dev))
+    refs = [t.float().requires_grad_(True) for t in (q, k, v)]
+    ref = O.sparse_attention_ref(*refs, mask)
+    ref.backward(w.float())
+    assert torch.allclose(out.float().cpu(), ref.detach(), atol=1e-2, rtol=1e-2)
+    for got, want in zip(leaves, refs):
+        assert got.grad.shape == want.grad.shape
+        bound = 1e-4 + 1e-2 * want.grad.abs().max() + 1e-2 * want.grad.abs()
+        assert ((got.grad.float().cpu() - want.grad).abs() <= bound).all()
+    inf = sa.sparse_attention_func(q.to(dev), k.to(dev), v.to(dev), mask.to(dev))
+    assert torch.equal(inf, out.detach())
