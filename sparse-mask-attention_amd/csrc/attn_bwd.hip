@@ -1,4 +1,4 @@
-// Masked-attention backward for gfx950 (MI355X), head_dim 64, fp16 / bf16, fp32 accumulate.
+// Masked-attention backward for gfx950 (MI355X), head_dim 64 or 128, fp16 / bf16, fp32 accumulate.
 //
 // The reference declares a backward launcher (csrc/sparse_attention.h:57-64) and its Python API
 // calls sparse_attn_cuda.backward (python/sparse_attention.py:91-94), but neither was ever

@@ -1,4 +1,4 @@
-// Fused masked-attention forward for gfx950 (MI355X), head_dim 64, fp16 / bf16, fp32 accumulate.
+// Fused masked-attention forward for gfx950 (MI355X), head_dim 64 or 128, fp16 / bf16, fp32 accumulate.
 //
 // Stands in for sparse_attn_wmma_full_fp16 (csrc/sparse_attention.cu:82-412 of the reference) and
 // for its scalar bf16 kernel (csrc/sparse_attention.cu:418-543); the design below is specific to
@@ -35,6 +35,9 @@
 //                 when its first finite score lies below the window; probabilities stay <= 2^8.
 //   skipping    = a wavefront whose own 32 x 64 block of mask bits is empty skips its GEMMs and its
 //                 softmax for that tile (the tile itself is still copied, see the main loop).
+//   head dim    = the description above is for 64.  128 runs the same code on two column halves of
+//                 64 (see Cfg below): twice the MFMAs per tile for the same softmax work, a ring of
+//                 two stages and two work-groups per CU.
 #include <type_traits>
 
 #include "attn_common.h"
