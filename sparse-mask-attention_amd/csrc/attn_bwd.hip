@@ -55,8 +55,6 @@ template <int NH> struct Cfg {
     static constexpr int LDS_BYTES = OFF_LUT + 256;
 };
 
-__device__ __forceinline__ int bitrev3(int f) { return ((f & 1) << 2) | (f & 2) | (f >> 2); }
-
 // Per-lane constants of the tile copies: wave w copies row blocks 2w and 2w+1 (8 rows each) of a
 // 64-row tile; lane i fills LDS chunk (row 8*blk + i/8, position i%8) with global chunk
 // position ^ bitrev3((row >> 1) & 7).
@@ -135,55 +133,10 @@ __device__ __forceinline__ TileRead make_tile_read(int lane)
     return r;
 }
 
-// XCD-aware renumbering of the work-groups (the 8 XCDs take them round-robin): each XCD owns a
-// contiguous range of (b,h) pairs, so the tiles of a head are fetched into one L2 only.
-__device__ __forceinline__ int renumber_block()
-{
-    const int total = gridDim.x, bid = blockIdx.x;
-    const int xcd = bid & 7, j = bid >> 3;
-    const int base = total >> 3, rem = total & 7;
-    return xcd * base + (xcd < rem ? xcd : rem) + j;
-}
-
 // 16 bytes (8 elements) of row `row` (row stride sn elements) at element offset `col`.
 __device__ __forceinline__ u32x4 load_frag(const uint16_t *mat, int sn, int row, int col)
 {
     return *reinterpret_cast<const u32x4 *>(mat + (size_t)row * sn + col);
-}
-
-// Transposed store of a 32 x 64 accumulator block (acc[dblk][4g+j] = value(row l32, column
-// 32dblk + 8g + 4hh + j), acc = {acc0, acc1}) times `mult`, through 4 KiB of wave-private LDS, as
-// whole 128-byte pieces of rows (dst_row0: first row, first of the 64 columns; sn: row stride in
-// elements).
-template <bool BF16>
-__device__ __forceinline__ void store_block(const f32x16 &acc0, const f32x16 &acc1, float mult, uint32_t lds_wave,
-                                            uint16_t *dst_row0, int sn, int row0, int N, int lane)
-{
-    const f32x16 acc[2] = {acc0, acc1};
-    using E = Elem<BF16>;
-    const int l32 = lane & 31, hh = lane >> 5;
-    const uint32_t wrow = lds_wave + l32 * 128 + hh * 8;
-    const int fo = (l32 >> 1) & 7;
-#pragma unroll
-    for (int dblk = 0; dblk < 2; ++dblk)
-#pragma unroll
-        for (int g = 0; g < 4; ++g) {
-            const u32x2 o = {E::pack2_rne(acc[dblk][4 * g + 0] * mult, acc[dblk][4 * g + 1] * mult),
-                             E::pack2_rne(acc[dblk][4 * g + 2] * mult, acc[dblk][4 * g + 3] * mult)};
-            *(LDS_PTR(u32x2))(uintptr_t)(wrow + (((4 * dblk + g) ^ fo) << 4)) = o;
-        }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int row = 8 * j + (lane >> 3), pos = lane & 7;
-        const u32x4 v = lds_read_b128(lds_wave + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
-        if (row0 + row < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst_row0 + (size_t)row * sn + pos * 8));
-    }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 
 // ------------------------------------------------------------------------------------------------

@@ -83,6 +83,21 @@ template <> struct Elem<true> {
     static constexpr float TERM_MAX = 3.0e38f;
 };
 
+// Bit reversal of a 3-bit value: the chunk swizzle of tiles that are read both by rows and transposed.
+__device__ __forceinline__ int bitrev3(int f) { return ((f & 1) << 2) | (f & 2) | (f >> 2); }
+
+// XCD-aware renumbering of the work-groups.  They are handed to the 8 XCDs round-robin by linear
+// id; the number returned gives each XCD (own L2) a contiguous range of (b,h) pairs, with the
+// tiles of one (b,h) dispatched next to each other: the matrices of a head are then fetched into
+// one L2 only.
+__device__ __forceinline__ int renumber_block()
+{
+    const int total = gridDim.x, bid = blockIdx.x;
+    const int xcd = bid & 7, j = bid >> 3;
+    const int base = total >> 3, rem = total & 7;
+    return xcd * base + (xcd < rem ? xcd : rem) + j;
+}
+
 // max / sum of a value with its partner in the other lane half (lane l <-> lane l ^ 32).
 // v_permlane32_swap(a, b) leaves {own a | partner's b, partner's a | own b} in lanes < 32 | >= 32.
 __device__ __forceinline__ float xhalf_max(float x) {
@@ -134,6 +149,42 @@ __device__ __forceinline__ void async_copy_b32_at(uint32_t lds_base, const void 
                  :: "s"(lds_base), "v"(voff), "s"(base), "n"(OFF) : "memory", "scc");
 }
 #define WAIT_VMCNT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
+
+
+// Transposed store of a 32 x 64 accumulator block (acc[dblk][4g+j] = value(row l32, column
+// 32dblk + 8g + 4hh + j), acc = {acc0, acc1}) times `mult`, through 4 KiB of wave-private LDS, as
+// whole 128-byte pieces of rows (dst_row0: first row, first of the 64 columns; sn: row stride in
+// elements).
+template <bool BF16>
+__device__ __forceinline__ void store_block(const f32x16 &acc0, const f32x16 &acc1, float mult, uint32_t lds_wave,
+                                            uint16_t *dst_row0, int sn, int row0, int N, int lane)
+{
+    const f32x16 acc[2] = {acc0, acc1};
+    using E = Elem<BF16>;
+    const int l32 = lane & 31, hh = lane >> 5;
+    const uint32_t wrow = lds_wave + l32 * 128 + hh * 8;
+    const int fo = (l32 >> 1) & 7;
+#pragma unroll
+    for (int dblk = 0; dblk < 2; ++dblk)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            const u32x2 o = {E::pack2_rne(acc[dblk][4 * g + 0] * mult, acc[dblk][4 * g + 1] * mult),
+                             E::pack2_rne(acc[dblk][4 * g + 2] * mult, acc[dblk][4 * g + 3] * mult)};
+            *(LDS_PTR(u32x2))(uintptr_t)(wrow + (((4 * dblk + g) ^ fo) << 4)) = o;
+        }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int row = 8 * j + (lane >> 3), pos = lane & 7;
+        const u32x4 v = lds_read_b128(lds_wave + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
+        if (row0 + row < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst_row0 + (size_t)row * sn + pos * 8));
+    }
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 
 }  // namespace
 }  // namespace sma

@@ -89,16 +89,7 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31, hh = lane >> 5;
 
-    // Work-groups are handed to the 8 XCDs round-robin by linear id.  Renumber so that each XCD
-    // (own L2) owns a contiguous range of (b,h) pairs and the query tiles of one (b,h) are
-    // dispatched next to each other: K and V of a head are then fetched into one L2 only.
-    int nid;
-    {
-        const int total = gridDim.x, bid = blockIdx.x;
-        const int xcd = bid & 7, j = bid >> 3;
-        const int base = total >> 3, rem = total & 7;
-        nid = xcd * base + (xcd < rem ? xcd : rem) + j;
-    }
+    const int nid = renumber_block();
     const int bh = (int)fastdiv((uint32_t)nid, a.div_qtiles);
     const int qt = nid - bh * a.qtiles;
     const int N = a.N, nw = (N + 31) >> 5;
@@ -143,7 +134,7 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
         const int row = 8 * (2 * wave + j) + (lane >> 3);
         const int pos = lane & 7;
         const int f = (row >> 1) & 7;
-        const int fr = ((f & 1) << 2) | (f & 2) | (f >> 2);
+        const int fr = bitrev3(f);
         // row pitches are below 2^24 bytes (checked by the C-ABI layer): full-rate 24-bit multiplies
         kv_voff[0][j] = __umul24(row, k_rb) + ((pos ^ f) << 4);
         kv_voff[1][j] = __umul24(row, v_rb) + ((pos ^ fr) << 4);
@@ -207,7 +198,7 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
         for (int x = 0; x < 2; ++x) {
             const int row = 8 * x + r3;
             const int f = (row >> 1) & 7;
-            const int fr = ((f & 1) << 2) | (f & 2) | (f >> 2);
+            const int fr = bitrev3(f);
 #pragma unroll
             for (int dblk = 0; dblk < 2; ++dblk) {
                 const int chunk = 4 * dblk + 2 * G + ((i16 & 3) >> 1);
@@ -432,41 +423,18 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
     // out = O / l.  The accumulator layout gives a lane 8-byte pieces of one row; written as they
     // are, a store instruction would touch 32 different 128-byte rows.  Each wave therefore
     // transposes its 32 x 64 block (one per column half) through 4 KiB of LDS (K/V stage 0, free
-    // after a barrier; chunks XOR-swizzled as for K) and stores whole 128-byte pieces of rows: 8 lanes
-    // x 16 B per row, 8 rows per instruction.
+    // after a barrier) and stores whole 128-byte pieces of rows, non-temporally: the output is not
+    // read again here and should not displace K, V and the mask.
     const float l_tot = xhalf_sum(l_run);
     const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
     __syncthreads();              // every wave is done reading the K/V stages
     {
-        const uint32_t obase = lds0 + wave * 4096;           // + 16 KiB for the second column half
-        const uint32_t wrow = obase + l32 * 128 + hh * 8;
-        const int fo = (l32 >> 1) & 7;
-#pragma unroll
-        for (int b = 0; b < 2 * NH; ++b)
-#pragma unroll
-            for (int g = 0; g < 4; ++g) {
-                const uint32_t lo = (uint32_t)E::cvt1(oacc[b][4 * g + 0] * inv) |
-                                    ((uint32_t)E::cvt1(oacc[b][4 * g + 1] * inv) << 16);
-                const uint32_t hi = (uint32_t)E::cvt1(oacc[b][4 * g + 2] * inv) |
-                                    ((uint32_t)E::cvt1(oacc[b][4 * g + 3] * inv) << 16);
-                const u32x2 o = {lo, hi};
-                *(LDS_PTR(u32x2))(uintptr_t)(wrow + (b >> 1) * 16384 + (((4 * (b & 1) + g) ^ fo) << 4)) = o;
-            }
-        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-        __builtin_amdgcn_wave_barrier();
-        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         const int row0 = qt * BM + wave * 32;
         uint16_t *ob = slab(a.out, bi, hi) + (size_t)row0 * o_sn;
 #pragma unroll
         for (int half = 0; half < NH; ++half)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int row = 8 * j + (lane >> 3), pos = lane & 7;
-                const u32x4 v = lds_read_b128(obase + half * 16384 + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
-                // non-temporal: the output is not read again here and should not displace K, V and the mask
-                if (row0 + row < N)
-                    __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(ob + (size_t)row * o_sn + half * HD + pos * 8));
-            }
+            store_block<BF16>(oacc[2 * half], oacc[2 * half + 1], inv, lds0 + wave * 4096 + half * 16384,
+                              ob + half * HD, (int)o_sn, row0, N, lane);
     }
     if (qrow < N) {
         if (a.lse != nullptr && hh == 0) {
