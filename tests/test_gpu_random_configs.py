@@ -1,0 +1,90 @@
+"""Seeded random configurations of the whole operator (forward and backward through the strided
+C entry points) against the oracle: head dim, dtype, extents, ragged lengths, layouts, shared masks,
+mask structure and scale are drawn together, so that combinations no hand-written case names are
+exercised.  Same bars as the dedicated tests at the API's scale 1/sqrt(D); a scale s times larger
+sharpens the softmax and multiplies the effect of the 16-bit rounding of the inputs and of the
+pre-scaled q, so the absolute and relative bars are multiplied by max(1, s) as well."""
+import math
+import random
+
+import pytest
+import torch
+
+import _capi
+from oracle import sma_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+RTOL = {torch.float16: 1e-2, torch.bfloat16: 2e-2}
+
+
+def _layout(t, kind, dev):
+    """Device tensor with the values of t ([B,H,N,D]) stored in the given layout, viewed [B,H,N,D]."""
+    td = t.to(dev)
+    if kind == "dense":
+        return td
+    if kind == "bnhd":
+        return td.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3)
+    if kind == "hbnd":
+        return td.permute(1, 0, 2, 3).contiguous().permute(1, 0, 2, 3)
+    if kind == "padded":
+        store = torch.zeros(*t.shape[:3], t.shape[3] + 24, dtype=t.dtype, device=dev)
+        store[..., :t.shape[3]] = td
+        return store[..., :t.shape[3]]
+    raise ValueError(kind)
+
+
+def _mask(rng, g, Bm, Hm, N):
+    kind = rng.choice(["random", "random", "dense", "causal", "block", "sparse_rows"])
+    if kind == "random":
+        return torch.rand(Bm, Hm, N, N, generator=g) < rng.choice([0.05, 0.25, 0.6])
+    if kind == "dense":
+        return torch.ones(Bm, Hm, N, N, dtype=torch.bool)
+    if kind == "causal":
+        return torch.tril(torch.ones(N, N, dtype=torch.bool)).expand(Bm, Hm, N, N).contiguous()
+    if kind == "block":
+        nb = -(-N // 32)
+        blocks = torch.rand(Bm, Hm, nb, nb, generator=g) < 0.3
+        return blocks.repeat_interleave(32, 2).repeat_interleave(32, 3)[:, :, :N, :N].contiguous()
+    m = torch.rand(Bm, Hm, N, N, generator=g) < 0.3
+    m[:, :, torch.rand(N, generator=g) < 0.3, :] = False          # many rows keep nothing
+    return m
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_configuration(dev, seed):
+    rng = random.Random(seed)
+    g = torch.Generator().manual_seed(seed)
+    D = rng.choice([64, 128])
+    dtype = rng.choice([torch.float16, torch.bfloat16])
+    B, H = rng.choice([(1, 1), (1, 3), (2, 2), (3, 1)])
+    N = rng.choice([1, 7, 32, 63, 64, 65, 100, 127, 128, 129, 191, 192, 250, 320, 401])
+    Bm, Hm = rng.choice([(B, H), (B, H), (1, 1), (B, 1), (1, H)])
+    scale = rng.choice([None, None, 0.05, 0.3, -0.2])
+    layouts = [rng.choice(["dense", "bnhd", "hbnd", "padded"]) for _ in range(8)]
+    q, k, v, do = [torch.randn(B, H, N, D, generator=g).to(dtype) for _ in range(4)]
+    mask = _mask(rng, g, Bm, Hm, N)
+    tag = f"seed {seed}: D{D} {dtype} B{B} H{H} N{N} mask[{Bm},{Hm}] scale {scale} layouts {layouts}"
+    print(tag, flush=True)
+
+    qd, kd, vd, dod = (_layout(t, l, dev) for t, l in zip((q, k, v, do), layouts[:4]))
+    packed = _capi.pack_mask(mask.to(dev))
+    assert torch.equal(packed.cpu(), torch.from_numpy(O.pack_mask_ref(mask)))
+    out_view = _layout(torch.full((B, H, N, D), float("nan"), dtype=dtype), layouts[4], dev)
+    out, lse = _capi.attn_fwd_strided(qd, kd, vd, packed, out=out_view, scale=scale, want_lse=True)
+    grads = tuple(_layout(torch.full((B, H, N, D), float("nan"), dtype=dtype), l, dev) for l in layouts[5:8])
+    dq, dk, dv, _ = _capi.attn_bwd_strided(dod, qd, kd, vd, out, lse, packed, grads=grads, scale=scale)
+    torch.cuda.synchronize()
+
+    full = mask.expand(B, H, N, N)
+    sharp = max(1.0, abs(scale) * math.sqrt(D)) if scale is not None else 1.0
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), full, scale=scale)
+    assert torch.allclose(out.float().cpu(), ref, atol=1e-2 * sharp, rtol=RTOL[dtype] * sharp), tag
+    empty = ~full.any(dim=-1)
+    assert (out.cpu()[empty] == 0).all() and (lse.cpu()[empty] == -math.inf).all(), tag
+    refs = O.sparse_attention_bwd_ref(q.float(), k.float(), v.float(), full, do.float(), scale=scale)
+    for name, got, want in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
+        got = got.float().cpu()
+        assert torch.isfinite(got).all(), f"{name} {tag}"
+        bound = 1e-4 + sharp * (1e-2 * want.abs().max() + RTOL[dtype] * want.abs())
+        assert ((got - want).abs() <= bound).all(), f"{name} {tag}: max err {(got - want).abs().max():.3e}"
