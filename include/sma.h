@@ -22,7 +22,7 @@ extern "C" {
 #define SMA_OK                 0
 #define SMA_ERR_NULL_POINTER  -1   /* a required pointer is NULL */
 #define SMA_ERR_BAD_SHAPE     -2   /* a negative extent, or an extent beyond the 32-bit index range */
-#define SMA_ERR_HEAD_DIM      -3   /* head_dim other than 64 or 128 */
+#define SMA_ERR_HEAD_DIM      -3   /* head_dim other than 32, 64 or 128 */
 #define SMA_ERR_DTYPE         -4   /* dtype other than SMA_DTYPE_F16 / SMA_DTYPE_BF16 */
 #define SMA_ERR_SCALE         -5   /* scale is NaN or infinite */
 #define SMA_ERR_LAUNCH        -6   /* the HIP runtime refused the launch (hipGetLastError) */
@@ -53,7 +53,7 @@ int sma_pack_mask(const uint8_t *mask, uint32_t *packed, int B, int H, int N, vo
 
 /* Fused masked attention forward:  out = softmax_row(mask ? (q k^T) * scale : -inf) v.
  *
- *   q, k, v      [B,H,N,D] fp16 or bf16 (dtype), D must be 64 (the reference's only head dim) or 128
+ *   q, k, v      [B,H,N,D] fp16 or bf16 (dtype), D = 64 (the reference's only head dim), 32 or 128
  *   mask_packed  uint32 [B,H,N,ceil(N/32)] in the sma_pack_mask format (pad bits are ignored)
  *   out          [B,H,N,D], same dtype; every element is written
  *   lse          NULL, or float [B,H,N]: natural-log-sum-exp of the kept scaled scores of each
@@ -74,7 +74,7 @@ int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *ma
 
 /* Masked attention backward:  given dout = dLoss/dout, the gradients with respect to q, k and v.
  *
- *   dout, q, k, v, out  [B,H,N,D] fp16 or bf16 (dtype), D 64 or 128; out and lse are the results
+ *   dout, q, k, v, out  [B,H,N,D] fp16 or bf16 (dtype), D = 32, 64 or 128; out and lse are the results
  *                       of sma_attn_fwd on the same q, k, v, mask_packed and scale
  *   lse                 float [B,H,N] as written by sma_attn_fwd (-inf for rows that keep no key)
  *   mask_packed         uint32 [B,H,N,ceil(N/32)]

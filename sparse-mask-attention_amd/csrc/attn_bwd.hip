@@ -1,4 +1,4 @@
-// Masked-attention backward for gfx950 (MI355X), head_dim 64 or 128, fp16 / bf16, fp32 accumulate.
+// Masked-attention backward for gfx950 (MI355X), head_dim 32, 64 or 128, fp16 / bf16, fp32 accumulate.
 //
 // The reference declares a backward launcher (csrc/sparse_attention.h:57-64) and its Python API
 // calls sparse_attn_cuda.backward (python/sparse_attention.py:91-94), but neither was ever
@@ -30,7 +30,9 @@
 // as two 64-column tiles, the products that contract over the head dim (S, dP) run over both
 // halves, the others (dQ, dK, dV) fill one pair of accumulators per half.  The dK/dV kernel would
 // need 128 accumulator registers for that; it is therefore launched twice, once for dK and once
-// for dV (S is formed in both).
+// for dV (S is formed in both).  Head dim 32 uses half a tile: the copies fill the upper half of
+// every LDS row with a second copy of the lower half (global chunk index & 3), which is never read;
+// contractions over the head dim take two MFMA steps and the outputs have one 32-column block.
 #include "attn_common.h"
 
 namespace sma {
@@ -62,7 +64,7 @@ struct TileCopy {
     uint32_t chunk[2];      // byte offset of the lane's global chunk inside its row
     int row[2];
 };
-__device__ __forceinline__ TileCopy make_tile_copy(int wave, int lane)
+__device__ __forceinline__ TileCopy make_tile_copy(int wave, int lane, int chunk_mask)
 {
     TileCopy c;
 #pragma unroll
@@ -70,7 +72,7 @@ __device__ __forceinline__ TileCopy make_tile_copy(int wave, int lane)
         const int row = 8 * (2 * wave + j) + (lane >> 3);
         const int pos = lane & 7;
         c.row[j] = row;
-        c.chunk[j] = (uint32_t)((pos ^ bitrev3((row >> 1) & 7)) << 4);
+        c.chunk[j] = (uint32_t)(((pos ^ bitrev3((row >> 1) & 7)) & chunk_mask) << 4);
     }
     return c;
 }
@@ -142,10 +144,14 @@ __device__ __forceinline__ u32x4 load_frag(const uint16_t *mat, int sn, int row,
 // ------------------------------------------------------------------------------------------------
 // dQ (and delta)
 // ------------------------------------------------------------------------------------------------
-template <bool BF16, int NH>
-__global__ __launch_bounds__(NTHREADS, NH == 1 ? 3 : 2) void attn_bwd_dq_kernel(const AttnBwdArgs a)
+template <bool BF16, int HDIM>
+__global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_bwd_dq_kernel(const AttnBwdArgs a)
 {
     using E = Elem<BF16>;
+    constexpr int NH = HDIM == 128 ? 2 : 1;       // 64-column tiles per matrix
+    constexpr int KS = HDIM / 16;                 // MFMA steps of a contraction over the head dim
+    constexpr int OB = HDIM / 32;                 // 32-column accumulator blocks of an output
+    constexpr int CHM = HDIM == 32 ? 3 : 7;       // 16-byte chunks per global row, minus one
     using C = Cfg<NH>;
     constexpr int STAGE_BYTES = C::STAGE_BYTES, OFF_AUX = C::OFF_AUX, OFF_LUT = C::OFF_LUT;
     __shared__ __attribute__((aligned(1024))) unsigned char smem[C::LDS_BYTES];
@@ -171,10 +177,10 @@ __global__ __launch_bounds__(NTHREADS, NH == 1 ? 3 : 2) void attn_bwd_dq_kernel(
     // ---- this lane's query row: q^T and dO^T fragments (B operands), delta, lse ----
     const int qrow = qt * BM + wave * 32 + l32;
     const int qr = qrow < N ? qrow : N - 1;
-    u32x4 qf[4 * NH], dof[4 * NH];
+    u32x4 qf[KS], dof[KS];
     float delta = 0.f;
 #pragma unroll
-    for (int s = 0; s < 4 * NH; ++s) {
+    for (int s = 0; s < KS; ++s) {
         const int col = 16 * s + 8 * hh;
         u32x4 tq = load_frag(qb, a.q.sn, qr, col);
         const u32x4 td = load_frag(dob, a.dout.sn, qr, col);
@@ -197,7 +203,7 @@ __global__ __launch_bounds__(NTHREADS, NH == 1 ? 3 : 2) void attn_bwd_dq_kernel(
     const float L = (qrow >= N || lse_row == -__builtin_inff()) ? __builtin_inff() : lse_row * LOG2E;
 
     // ---- copies ----
-    const TileCopy tc = make_tile_copy(wave, lane);
+    const TileCopy tc = make_tile_copy(wave, lane, CHM);
     const TileRead tr = make_tile_read(lane);
     const int mrow = qt * BM + wave * 32 + (lane >> 1);
     const uint32_t m_voff = (uint32_t)(((size_t)(mrow < N ? mrow : N - 1) * nw + (lane & 1)) * 4);
@@ -212,9 +218,9 @@ __global__ __launch_bounds__(NTHREADS, NH == 1 ? 3 : 2) void attn_bwd_dq_kernel(
     if (tid < 64)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
 
-    f32x16 oacc[2 * NH];                // [2 * half + dblk]: 32 columns of dQ each
+    f32x16 oacc[OB];                    // [2 * half + dblk]: 32 columns of dQ each
 #pragma unroll
-    for (int b = 0; b < 2 * NH; ++b)
+    for (int b = 0; b < OB; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[b][i] = 0.f;
     const uint32_t lut_addr = lds0 + OFF_LUT;
@@ -249,7 +255,7 @@ __global__ __launch_bounds__(NTHREADS, NH == 1 ? 3 : 2) void attn_bwd_dq_kernel(
                 }
             }
 #pragma unroll
-            for (int s = 0; s < 4 * NH; ++s) {
+            for (int s = 0; s < KS; ++s) {
                 const uint32_t ra = tr.rowaddr[s & 3] + so + (s >> 2) * TILE_BYTES + 4096 * blk;
                 sacc = E::mfma(lds_read_b128(ra), qf[s], sacc);
                 dacc = E::mfma(lds_read_b128(ra + C::OFF_B), dof[s], dacc);
@@ -272,7 +278,7 @@ __global__ __launch_bounds__(NTHREADS, NH == 1 ? 3 : 2) void attn_bwd_dq_kernel(
                 const u32x4 pv = {pb[blk][u][0], pb[blk][u][1], pb[blk][u][2], pb[blk][u][3]};
                 const uint32_t off = so + 4096 * blk + 2048 * u;
 #pragma unroll
-                for (int b = 0; b < 2 * NH; ++b) {
+                for (int b = 0; b < OB; ++b) {
                     const uint32_t ko = off + (b >> 1) * TILE_BYTES;
                     const u32x2 lo = lds_read_tr16_b64(tr.traddr[b & 1][0] + ko);
                     const u32x2 hi = lds_read_tr16_b64(tr.traddr[b & 1][1] + ko);
@@ -285,10 +291,15 @@ __global__ __launch_bounds__(NTHREADS, NH == 1 ? 3 : 2) void attn_bwd_dq_kernel(
     __syncthreads();              // every wave is done reading the stages
     const int row0 = qt * BM + wave * 32;
     if (row0 < N) {
+        uint16_t *dst = slab(a.dq, bi, hi) + (size_t)row0 * a.dq.sn;
+        if constexpr (HDIM == 32) {
+            store_block<BF16, 32>(oacc[0], oacc[0], a.scale, lds0 + wave * 4096, dst, a.dq.sn, row0, N, lane);
+        } else {
 #pragma unroll
-        for (int half = 0; half < NH; ++half)
-            store_block<BF16>(oacc[2 * half], oacc[2 * half + 1], a.scale, lds0 + wave * 4096,
-                              slab(a.dq, bi, hi) + (size_t)row0 * a.dq.sn + half * HD, a.dq.sn, row0, N, lane);
+            for (int half = 0; half < NH; ++half)
+                store_block<BF16>(oacc[2 * half], oacc[2 * half + 1], a.scale, lds0 + wave * 4096,
+                                  dst + half * HD, a.dq.sn, row0, N, lane);
+        }
     }
 }
 
@@ -297,10 +308,14 @@ __global__ __launch_bounds__(NTHREADS, NH == 1 ? 3 : 2) void attn_bwd_dq_kernel(
 // ------------------------------------------------------------------------------------------------
 // DK / DV: which of the two gradients this instance produces (both for head dim 64; one per launch
 // for head dim 128, where both sets of accumulators do not fit the register file).
-template <bool BF16, int NH, bool DK, bool DV>
+template <bool BF16, int HDIM, bool DK, bool DV>
 __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwdArgs a)
 {
     using E = Elem<BF16>;
+    constexpr int NH = HDIM == 128 ? 2 : 1;
+    constexpr int KS = HDIM / 16;
+    constexpr int OB = HDIM / 32;
+    constexpr int CHM = HDIM == 32 ? 3 : 7;
     using C = Cfg<NH>;
     constexpr int STAGE_BYTES = C::STAGE_BYTES, OFF_AUX = C::OFF_AUX;
     __shared__ __attribute__((aligned(1024))) unsigned char smem[C::LDS_BYTES];
@@ -331,9 +346,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     const int kr = key < N ? key : N - 1;
     const uint32_t key_ok = key < N ? 0xffffffffu : 0u;
     const int wi = (key0 >> 5) < nw ? (key0 >> 5) : nw - 1;     // this wave's mask word of a row
-    u32x4 kf[4 * NH], vf[DK ? 4 * NH : 1];
+    u32x4 kf[KS], vf[DK ? KS : 1];
 #pragma unroll
-    for (int s = 0; s < 4 * NH; ++s) {
+    for (int s = 0; s < KS; ++s) {
         const int col = 16 * s + 8 * hh;
         u32x4 tk = load_frag(kb, a.k.sn, kr, col);
         if constexpr (DK) vf[s] = load_frag(vb, a.v.sn, kr, col);
@@ -347,7 +362,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     }
 
     // ---- copies: Q tile, dO tile; per wave its mask word of the 64 rows; lse (wave 0), delta (wave 1)
-    const TileCopy tc = make_tile_copy(wave, lane);
+    const TileCopy tc = make_tile_copy(wave, lane, CHM);
     const TileRead tr = make_tile_read(lane);
     auto issue = [&](int t, int st) {
         const int r0 = t * BN;
@@ -361,9 +376,9 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     };
     issue(0, 0);
 
-    f32x16 dkacc[DK ? 2 * NH : 1], dvacc[DV ? 2 * NH : 1];      // [2 * half + dblk]: 32 columns each
+    f32x16 dkacc[DK ? OB : 1], dvacc[DV ? OB : 1];      // [2 * half + dblk]: 32 columns each
 #pragma unroll
-    for (int b = 0; b < 2 * NH; ++b)
+    for (int b = 0; b < OB; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             if constexpr (DK) dkacc[b][i] = 0.f;
@@ -404,11 +419,11 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
 #pragma unroll
             for (int i = 0; i < 16; ++i) { sacc[i] = 0.f; dacc[i] = 0.f; }
 #pragma unroll
-            for (int s = 0; s < 4 * NH; ++s)
+            for (int s = 0; s < KS; ++s)
                 sacc = E::mfma(lds_read_b128(tr.rowaddr[s & 3] + so + (s >> 2) * TILE_BYTES + 4096 * blk), kf[s], sacc);
             if constexpr (DK) {
 #pragma unroll
-                for (int s = 0; s < 4 * NH; ++s)
+                for (int s = 0; s < KS; ++s)
                     dacc = E::mfma(lds_read_b128(tr.rowaddr[s & 3] + so + C::OFF_B + (s >> 2) * TILE_BYTES + 4096 * blk),
                                    vf[s], dacc);
             }
@@ -445,7 +460,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
                 const u32x4 bs = {ps[u][0], ps[u][1], ps[u][2], ps[u][3]};
                 const uint32_t off = so + 4096 * blk + 2048 * u;
 #pragma unroll
-                for (int b = 0; b < 2 * NH; ++b) {
+                for (int b = 0; b < OB; ++b) {
                     const uint32_t ho = off + (b >> 1) * TILE_BYTES;
                     if constexpr (DK) {                              // dK^T += Q^T dS
                         const u32x2 qlo = lds_read_tr16_b64(tr.traddr[b & 1][0] + ho);
@@ -466,14 +481,21 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     WAIT_VMCNT(0);
     __syncthreads();
     if (wave_valid) {
+        uint16_t *dk_dst = slab(a.dk, bi, hi) + (size_t)key0 * a.dk.sn;
+        uint16_t *dv_dst = slab(a.dv, bi, hi) + (size_t)key0 * a.dv.sn;
+        if constexpr (HDIM == 32) {
+            if constexpr (DK) store_block<BF16, 32>(dkacc[0], dkacc[0], a.scale, lds0 + wave * 4096, dk_dst, a.dk.sn, key0, N, lane);
+            if constexpr (DV) store_block<BF16, 32>(dvacc[0], dvacc[0], 1.0f, lds0 + wave * 4096, dv_dst, a.dv.sn, key0, N, lane);
+        } else {
 #pragma unroll
-        for (int half = 0; half < NH; ++half) {
-            if constexpr (DK)
-                store_block<BF16>(dkacc[2 * half], dkacc[2 * half + 1], a.scale, lds0 + wave * 4096,
-                                  slab(a.dk, bi, hi) + (size_t)key0 * a.dk.sn + half * HD, a.dk.sn, key0, N, lane);
-            if constexpr (DV)
-                store_block<BF16>(dvacc[2 * half], dvacc[2 * half + 1], 1.0f, lds0 + wave * 4096,
-                                  slab(a.dv, bi, hi) + (size_t)key0 * a.dv.sn + half * HD, a.dv.sn, key0, N, lane);
+            for (int half = 0; half < NH; ++half) {
+                if constexpr (DK)
+                    store_block<BF16>(dkacc[2 * half], dkacc[2 * half + 1], a.scale, lds0 + wave * 4096,
+                                      dk_dst + half * HD, a.dk.sn, key0, N, lane);
+                if constexpr (DV)
+                    store_block<BF16>(dvacc[2 * half], dvacc[2 * half + 1], 1.0f, lds0 + wave * 4096,
+                                      dv_dst + half * HD, a.dv.sn, key0, N, lane);
+            }
         }
     }
 }
@@ -489,23 +511,31 @@ hipError_t launch_attn_bwd(const AttnBwdArgs &args, bool bf16, hipStream_t strea
     if (groups == 0) return hipSuccess;
     const dim3 grid((unsigned)groups), block(NTHREADS);
     // dQ first: it also fills the delta workspace that the dK/dV kernel reads (same stream).
-    if (a.D == HD) {
+    if (a.D == 2 * HD) {
         if (bf16) {
-            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 1>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 1, true, true>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 128>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 128, true, false>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 128, false, true>), grid, block, 0, stream, a);
         } else {
-            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 1>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 1, true, true>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 128>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 128, true, false>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 128, false, true>), grid, block, 0, stream, a);
+        }
+    } else if (a.D == HD) {
+        if (bf16) {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 64>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 64, true, true>), grid, block, 0, stream, a);
+        } else {
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 64>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 64, true, true>), grid, block, 0, stream, a);
         }
     } else {
         if (bf16) {
-            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 2>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 2, true, false>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 2, false, true>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 32>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 32, true, true>), grid, block, 0, stream, a);
         } else {
-            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 2>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 2, true, false>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 2, false, true>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 32>), grid, block, 0, stream, a);
+            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 32, true, true>), grid, block, 0, stream, a);
         }
     }
     return hipGetLastError();

@@ -151,11 +151,12 @@ __device__ __forceinline__ void async_copy_b32_at(uint32_t lds_base, const void 
 #define WAIT_VMCNT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
 
 
-// Transposed store of a 32 x 64 accumulator block (acc[dblk][4g+j] = value(row l32, column
-// 32dblk + 8g + 4hh + j), acc = {acc0, acc1}) times `mult`, through 4 KiB of wave-private LDS, as
-// whole 128-byte pieces of rows (dst_row0: first row, first of the 64 columns; sn: row stride in
-// elements).
-template <bool BF16>
+// Transposed store of a 32 x COLS accumulator block (COLS = 64: acc[dblk][4g+j] = value(row l32,
+// column 32dblk + 8g + 4hh + j) with acc = {acc0, acc1}; COLS = 32: acc0 only) times `mult`, through
+// 4 KiB of wave-private LDS, as whole 2*COLS-byte pieces of rows (dst_row0: first row, first of the
+// COLS columns; sn: row stride in elements).  Non-temporal stores: what is written is not read
+// again by the kernel and should not displace its inputs from the caches.
+template <bool BF16, int COLS = 64>
 __device__ __forceinline__ void store_block(const f32x16 &acc0, const f32x16 &acc1, float mult, uint32_t lds_wave,
                                             uint16_t *dst_row0, int sn, int row0, int N, int lane)
 {
@@ -165,7 +166,7 @@ __device__ __forceinline__ void store_block(const f32x16 &acc0, const f32x16 &ac
     const uint32_t wrow = lds_wave + l32 * 128 + hh * 8;
     const int fo = (l32 >> 1) & 7;
 #pragma unroll
-    for (int dblk = 0; dblk < 2; ++dblk)
+    for (int dblk = 0; dblk < COLS / 32; ++dblk)
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
             const u32x2 o = {E::pack2_rne(acc[dblk][4 * g + 0] * mult, acc[dblk][4 * g + 1] * mult),
@@ -175,9 +176,10 @@ __device__ __forceinline__ void store_block(const f32x16 &acc0, const f32x16 &ac
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    constexpr int LPR = COLS / 8;                 // lanes (16-byte chunks) per row
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int row = 8 * j + (lane >> 3), pos = lane & 7;
+    for (int j = 0; j < LPR / 2; ++j) {
+        const int row = (64 / LPR) * j + lane / LPR, pos = lane % LPR;
         const u32x4 v = lds_read_b128(lds_wave + row * 128 + ((pos ^ ((row >> 1) & 7)) << 4));
         if (row0 + row < N) __builtin_nontemporal_store(v, reinterpret_cast<u32x4 *>(dst_row0 + (size_t)row * sn + pos * 8));
     }

@@ -1,4 +1,4 @@
-// Fused masked-attention forward for gfx950 (MI355X), head_dim 64 or 128, fp16 / bf16, fp32 accumulate.
+// Fused masked-attention forward for gfx950 (MI355X), head_dim 32, 64 or 128, fp16 / bf16, fp32 accumulate.
 //
 // Stands in for sparse_attn_wmma_full_fp16 (csrc/sparse_attention.cu:82-412 of the reference) and
 // for its scalar bf16 kernel (csrc/sparse_attention.cu:418-543); the design below is specific to
@@ -37,7 +37,7 @@
 //                 softmax for that tile (the tile itself is still copied, see the main loop).
 //   head dim    = the description above is for 64.  128 runs the same code on two column halves of
 //                 64 (see Cfg below): twice the MFMAs per tile for the same softmax work, a ring of
-//                 two stages and two work-groups per CU.
+//                 two stages and two work-groups per CU.  32 uses half of every tile row.
 #include <type_traits>
 
 #include "attn_common.h"
@@ -52,11 +52,15 @@ constexpr int NTHREADS = 256;
 constexpr int TILE_BYTES = BN * HD * 2;          // 8 KiB, rows of 128 B
 constexpr float WINDOW_LOG2 = 8.0f;
 
-// Head dim 64 * NH.  A head dim of 128 is handled as two column halves of 64: K and V tiles are kept
-// in LDS as two 64-column tiles each (same row length, swizzles and read patterns as for 64), the
-// QK^T chain runs over both halves of K and q, and P multiplies each half of V into its own pair
-// of accumulators.  Its stage is twice as large, so the ring has two stages (copies one tile
-// ahead) and two work-groups share a CU.
+// Head dims (HDIM) other than 64 reuse the 64-column LDS tile with its 128-byte rows, swizzles and
+// read patterns:
+//   128  two column halves (NH = 2): K and V tiles are kept in LDS as two 64-column tiles each, the
+//        QK^T chain runs over both halves of K and q, and P multiplies each half of V into its own
+//        pair of accumulators.  A stage is twice as large, so the ring has two stages (copies one
+//        tile ahead) and two work-groups share a CU.
+//   32   half a tile: the copies fill the upper half of every LDS row with a second copy of the
+//        lower half (global chunk index & 3), which is never read; the QK^T chain has two steps
+//        instead of four and P multiplies one 32-column block of V.
 template <int NH> struct Cfg {
     static constexpr int NSTAGE = NH == 1 ? 3 : 2;
     static constexpr int WAVES_PER_SIMD = NH == 1 ? 3 : 2;
@@ -74,13 +78,17 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_
 // PACKED_ROWS: the rows of q, k, v and out follow each other without gaps (row stride 64), as in
 // contiguous tensors; the strides between heads and batch entries stay free.  A row stride known
 // at compile time measured 0.25 us less fixed cost per launch than the same value read at run time.
-template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int NH>
-__global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_kernel(const AttnArgs a)
+template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int HDIM>
+__global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD) void attn_fwd_kernel(const AttnArgs a)
 {
     using E = Elem<BF16>;
+    constexpr int NH = HDIM == 128 ? 2 : 1;       // 64-column tiles per matrix
+    constexpr int KS = HDIM / 16;                 // MFMA steps of the QK^T chain
+    constexpr int OB = HDIM / 32;                 // 32-column accumulator blocks of O
+    constexpr int CHM = HDIM == 32 ? 3 : 7;       // 16-byte chunks per global row, minus one
     using C = Cfg<NH>;
     constexpr int NSTAGE = C::NSTAGE, STAGE_BYTES = C::STAGE_BYTES, OFF_MASK = C::OFF_MASK, OFF_LUT = C::OFF_LUT;
-    constexpr int D = HD * NH;
+    constexpr int D = HDIM;
     __shared__ __attribute__((aligned(1024))) unsigned char smem[C::LDS_BYTES];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem;
 
@@ -136,8 +144,8 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
         const int f = (row >> 1) & 7;
         const int fr = bitrev3(f);
         // row pitches are below 2^24 bytes (checked by the C-ABI layer): full-rate 24-bit multiplies
-        kv_voff[0][j] = __umul24(row, k_rb) + ((pos ^ f) << 4);
-        kv_voff[1][j] = __umul24(row, v_rb) + ((pos ^ fr) << 4);
+        kv_voff[0][j] = __umul24(row, k_rb) + (((pos ^ f) & CHM) << 4);
+        kv_voff[1][j] = __umul24(row, v_rb) + (((pos ^ fr) & CHM) << 4);
     }
     const uint32_t kv_dst = lds0 + wave * 2048;
     auto issue_kv = [&](int t, auto stage_c) __attribute__((always_inline)) {
@@ -224,7 +232,7 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
             const int row = 8 * j + (lane >> 3);
             const int pos = lane & 7;
             const int lrow = row < last ? row : last;
-            const uint32_t voff = __umul24(lrow, q_rb) + ((pos ^ ((row >> 1) & 7)) << 4);
+            const uint32_t voff = __umul24(lrow, q_rb) + (((pos ^ ((row >> 1) & 7)) & CHM) << 4);
             async_copy_b128(dst + j * 1024, qsrc, voff);
             if constexpr (NH == 2) async_copy_b128(dst + 16384 + j * 1024, qsrc + HD, voff);
         }
@@ -235,7 +243,7 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
     // small LDS table for the mask: entry n (16 B) holds four floats, float j = (bit j of n) ? 0 : -inf
     if (tid < 64)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
-    const bool even_progress = NH == 1 && (int)blockIdx.x >= a.tail_start;
+    const bool even_progress = NH == 1 && (int)blockIdx.x >= a.tail_start;   // three work-groups per CU
     if (even_progress && T >= 4) __builtin_amdgcn_s_setprio(3);
     if constexpr (NSTAGE == 3) {
         if (T > 1) { issue_mask(1, integral_constant<int, 1>{}); issue_kv(1, integral_constant<int, 1>{}); }
@@ -245,9 +253,9 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
     }
     // ---- Q^T as MFMA B operands, scaled by scale*log2(e)/post_mul:
     //      lane holds query row l32, d = 16*s + 8*hh .. +7
-    u32x4 qf[4 * NH];
+    u32x4 qf[KS];
 #pragma unroll
-    for (int s = 0; s < 4 * NH; ++s) {
+    for (int s = 0; s < KS; ++s) {
         u32x4 t = lds_read_b128(kaddr[s & 3] + (NSTAGE - 1) * STAGE_BYTES + (s >> 2) * 16384 + wave * 4096);
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -259,9 +267,9 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
     }
 
     // ---- running state: one query row per lane; both lane halves hold the same ref ----
-    f32x16 oacc[2 * NH];                // [2 * half + dblk]: 32 columns each
+    f32x16 oacc[OB];                    // [2 * half + dblk]: 32 columns each
 #pragma unroll
-    for (int b = 0; b < 2 * NH; ++b)
+    for (int b = 0; b < OB; ++b)
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[b][i] = 0.f;
     float ref = 0.f;                    // reference point r, in accumulator units (log2 / pm)
@@ -310,7 +318,7 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
             sacc[1] = E::mfma(ones, refb, sacc[1]);
         }
 #pragma unroll
-        for (int s = 0; s < 4 * NH; ++s) {
+        for (int s = 0; s < KS; ++s) {
             const uint32_t ka = kaddr[s & 3] + so + (s >> 2) * TILE_BYTES;
             sacc[0] = E::mfma(lds_read_b128(ka), qf[s], sacc[0]);
             sacc[1] = E::mfma(lds_read_b128(ka + 4096), qf[s], sacc[1]);
@@ -338,7 +346,7 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
 #pragma unroll
             for (int i = 0; i < 16; ++i) {
 #pragma unroll
-                for (int b = 0; b < 2 * NH; ++b) oacc[b][i] *= alpha;
+                for (int b = 0; b < OB; ++b) oacc[b][i] *= alpha;
                 sacc[0][i] += delta; sacc[1][i] += delta;
             }
             rmax = top + delta;
@@ -370,7 +378,7 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
                 const u32x4 pv = {pb[blk][u][0], pb[blk][u][1], pb[blk][u][2], pb[blk][u][3]};
                 const uint32_t off = so + 4096 * blk + 2048 * u;
 #pragma unroll
-                for (int b = 0; b < 2 * NH; ++b) {
+                for (int b = 0; b < OB; ++b) {
                     const uint32_t voff = off + (b >> 1) * TILE_BYTES;
                     const u32x2 lo = lds_read_tr16_b64(vaddr[b & 1][0] + voff);
                     const u32x2 hi = lds_read_tr16_b64(vaddr[b & 1][1] + voff);
@@ -431,10 +439,14 @@ __global__ __launch_bounds__(NTHREADS, Cfg<NH>::WAVES_PER_SIMD) void attn_fwd_ke
     {
         const int row0 = qt * BM + wave * 32;
         uint16_t *ob = slab(a.out, bi, hi) + (size_t)row0 * o_sn;
+        if constexpr (HDIM == 32) {
+            store_block<BF16, 32>(oacc[0], oacc[0], inv, lds0 + wave * 4096, ob, (int)o_sn, row0, N, lane);
+        } else {
 #pragma unroll
-        for (int half = 0; half < NH; ++half)
-            store_block<BF16>(oacc[2 * half], oacc[2 * half + 1], inv, lds0 + wave * 4096 + half * 16384,
-                              ob + half * HD, (int)o_sn, row0, N, lane);
+            for (int half = 0; half < NH; ++half)
+                store_block<BF16>(oacc[2 * half], oacc[2 * half + 1], inv, lds0 + wave * 4096 + half * 16384,
+                                  ob + half * HD, (int)o_sn, row0, N, lane);
+        }
     }
     if (qrow < N) {
         if (a.lse != nullptr && hh == 0) {
@@ -476,26 +488,22 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     const bool postmul = a.post_mul != 1.0f;
     const int D = a.D;
     const bool packed = (int)a.q.sn == D && (int)a.k.sn == D && (int)a.v.sn == D && (int)a.out.sn == D;
-    if (D != HD) a.tail_start = (int)groups;                  // two work-groups per CU: nobody yields
+    if (D == 2 * HD) a.tail_start = (int)groups;              // two work-groups per CU: nobody yields
     void (*kernel)(const AttnArgs) = nullptr;
-    switch ((D == 2 * HD ? 8 : 0) | (bf16 ? 4 : 0) | (postmul ? 2 : 0) | (packed ? 1 : 0)) {
-    case 0: kernel = attn_fwd_kernel<false, false, false, 1>; break;
-    case 1: kernel = attn_fwd_kernel<false, false, true, 1>; break;
-    case 2: kernel = attn_fwd_kernel<false, true, false, 1>; break;
-    case 3: kernel = attn_fwd_kernel<false, true, true, 1>; break;
-    case 4: kernel = attn_fwd_kernel<true, false, false, 1>; break;
-    case 5: kernel = attn_fwd_kernel<true, false, true, 1>; break;
-    case 6: kernel = attn_fwd_kernel<true, true, false, 1>; break;
-    case 7: kernel = attn_fwd_kernel<true, true, true, 1>; break;
-    case 8: kernel = attn_fwd_kernel<false, false, false, 2>; break;
-    case 9: kernel = attn_fwd_kernel<false, false, true, 2>; break;
-    case 10: kernel = attn_fwd_kernel<false, true, false, 2>; break;
-    case 11: kernel = attn_fwd_kernel<false, true, true, 2>; break;
-    case 12: kernel = attn_fwd_kernel<true, false, false, 2>; break;
-    case 13: kernel = attn_fwd_kernel<true, false, true, 2>; break;
-    case 14: kernel = attn_fwd_kernel<true, true, false, 2>; break;
-    default: kernel = attn_fwd_kernel<true, true, true, 2>; break;
+    const int variant = (bf16 ? 4 : 0) | (postmul ? 2 : 0) | (packed ? 1 : 0);
+#define SMA_FWD_VARIANTS(HDIM)                                                          \
+    switch (variant) {                                                                 \
+    case 0: kernel = attn_fwd_kernel<false, false, false, HDIM>; break;                \
+    case 1: kernel = attn_fwd_kernel<false, false, true, HDIM>; break;                 \
+    case 2: kernel = attn_fwd_kernel<false, true, false, HDIM>; break;                 \
+    case 3: kernel = attn_fwd_kernel<false, true, true, HDIM>; break;                  \
+    case 4: kernel = attn_fwd_kernel<true, false, false, HDIM>; break;                 \
+    case 5: kernel = attn_fwd_kernel<true, false, true, HDIM>; break;                  \
+    case 6: kernel = attn_fwd_kernel<true, true, false, HDIM>; break;                  \
+    default: kernel = attn_fwd_kernel<true, true, true, HDIM>; break;                  \
     }
+    if (D == 32) { SMA_FWD_VARIANTS(32) } else if (D == 64) { SMA_FWD_VARIANTS(64) } else { SMA_FWD_VARIANTS(128) }
+#undef SMA_FWD_VARIANTS
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, a);
     return hipGetLastError();
 }

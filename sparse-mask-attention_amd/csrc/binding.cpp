@@ -11,7 +11,7 @@
 //
 // Differences, all on the safe side: `lse` may be None (the reference's own inference wrapper
 // passes None, python/sparse_attention.py:170-171); every tensor argument is checked (device,
-// dtype, shape, layout, head_dim 64 or 128) instead of only `q`; launches go to the current HIP
+// dtype, shape, layout, head_dim 32, 64 or 128) instead of only `q`; launches go to the current HIP
 // stream of q's device under a device guard; a failed launch raises RuntimeError.
 // q, k, v, out and the gradients need not be contiguous: any view whose last dimension is
 // contiguous and whose other strides are multiples of 8 elements is passed on with its strides
@@ -71,7 +71,7 @@ void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor
     const auto dt = q.scalar_type();
     TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "Unsupported dtype, need BF16 or FP16");
     const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
-    TORCH_CHECK(D == 64 || D == 128, "head_dim must be 64 or 128, got ", D);
+    TORCH_CHECK(D == 32 || D == 64 || D == 128, "head_dim must be 32, 64 or 128, got ", D);
     for (const torch::Tensor *t : {&k, &v, static_cast<const torch::Tensor *>(&out)}) {
         TORCH_CHECK(t->device() == q.device(), "q, k, v, out must be on the same device");
         TORCH_CHECK(t->scalar_type() == dt, "q, k, v, out must have the same dtype");
@@ -113,7 +113,7 @@ void backward(const torch::Tensor &dout, const torch::Tensor &q, const torch::Te
     const auto dt = q.scalar_type();
     TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "Unsupported dtype, need BF16 or FP16");
     const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
-    TORCH_CHECK(D == 64 || D == 128, "head_dim must be 64 or 128, got ", D);
+    TORCH_CHECK(D == 32 || D == 64 || D == 128, "head_dim must be 32, 64 or 128, got ", D);
     const torch::Tensor *all[8] = {&dout, &q, &k, &v, &out, &dq, &dk, &dv};
     const char *names[8] = {"dout", "q", "k", "v", "out", "dq", "dk", "dv"};
     sma_tensor d[8];

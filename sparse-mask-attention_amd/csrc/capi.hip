@@ -41,7 +41,7 @@ const char *sma_strerror(int code)
     case SMA_OK:               return "ok";
     case SMA_ERR_NULL_POINTER: return "a required pointer is NULL";
     case SMA_ERR_BAD_SHAPE:    return "bad shape: negative extent or index range exceeded";
-    case SMA_ERR_HEAD_DIM:     return "unsupported head_dim (64 or 128)";
+    case SMA_ERR_HEAD_DIM:     return "unsupported head_dim (32, 64 or 128)";
     case SMA_ERR_DTYPE:        return "unsupported dtype (need fp16 or bf16)";
     case SMA_ERR_SCALE:        return "scale must be finite";
     case SMA_ERR_LAUNCH:       return "HIP kernel launch failed";
@@ -98,7 +98,7 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
                          void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
-    if (D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
+    if (D != 32 && D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
     if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
     if (!isfinite(scale)) return SMA_ERR_SCALE;
     const long long BH = (long long)B * H;
@@ -106,6 +106,8 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
     if (!lse || !mask_packed || !delta_ws) return SMA_ERR_NULL_POINTER;
     const long long qtiles = (N + 127) / 128;
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
+    // a lane's byte offset into the packed mask of one (b,h) is a 32-bit register
+    if ((long long)N * ((N + 31) / 32) * 4 >= (1ll << 32)) return SMA_ERR_BAD_SHAPE;
     if (misaligned(mask_packed, 4) || misaligned(lse, 4) || misaligned(delta_ws, 4)) return SMA_ERR_ALIGNMENT;
     if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 
@@ -137,7 +139,7 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
                          int dtype, void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
-    if (D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
+    if (D != 32 && D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
     if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
     if (!isfinite(scale)) return SMA_ERR_SCALE;
     const long long BH = (long long)B * H;
@@ -145,6 +147,8 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
     if (!mask_packed) return SMA_ERR_NULL_POINTER;
     const long long qtiles = (N + 127) / 128;
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
+    // a lane's byte offset into the packed mask of one (b,h) is a 32-bit register
+    if ((long long)N * ((N + 31) / 32) * 4 >= (1ll << 32)) return SMA_ERR_BAD_SHAPE;
     if (misaligned(mask_packed, 4) || (lse && misaligned(lse, 4))) return SMA_ERR_ALIGNMENT;
     if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 

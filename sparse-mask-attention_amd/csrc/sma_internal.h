@@ -50,7 +50,7 @@ struct AttnArgs {
     Rows out;
     float *lse;                     // [BH, N] contiguous, or nullptr
     int BH, H, N;
-    int D;                          // head dim: 64 or 128
+    int D;                          // head dim: 32, 64 or 128
     int qtiles;                     // ceil(N / 128): query tiles (work-groups) per (b,h)
     FastDiv div_qtiles, div_H;      // filled in by the launcher
     // exp(scale * s) is evaluated as exp2(post_mul * (q_scale * q) . k): q is multiplied by
@@ -73,7 +73,7 @@ struct AttnBwdArgs {
     Rows dq, dk, dv;
     float *delta;                              // [BH, N] workspace: sum_d dout * out per query row
     int BH, H, N;
-    int D;                                     // head dim: 64 or 128
+    int D;                                     // head dim: 32, 64 or 128
     int qtiles;                                // ceil(N / 128)
     FastDiv div_qtiles, div_H;                 // filled in by the launcher
     float scale;                               // as given by the caller

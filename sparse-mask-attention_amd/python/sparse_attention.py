@@ -9,8 +9,8 @@ Mirrors ``python/sparse_attention.py`` of the reference (line numbers below refe
 * ``sparse_attention_ref``                  :24-42    the plain-PyTorch statement of the operator
 * ``generate_random_sparse_mask``           :204-211
 
-``q, k, v`` are ``[B, H, N, D]`` fp16 / bf16 tensors on an MI355X, D = 64 as in the reference or
-128 (other head dims up to 128 are zero-padded to the next of the two, see below) (fp32 inputs are computed in
+``q, k, v`` are ``[B, H, N, D]`` fp16 / bf16 tensors on an MI355X, D = 64 as in the reference, 32 or
+128 (other head dims up to 128 are zero-padded to the next of these, see below) (fp32 inputs are computed in
 bf16 and returned as fp32, as in the reference :140-142,151-152); ``mask`` is a bool
 ``[B, H, N, N]`` tensor, True = attend.  Query rows that attend to nothing give zeros.
 
@@ -28,8 +28,8 @@ What differs from the reference, on purpose:
 * ``mask`` may be ``[1, 1, N, N]``, ``[B, 1, N, N]`` or ``[1, H, N, N]``: it is packed once at that
   size and shared between batch entries / heads by the kernels (the reference needs the expanded
   ``[B, H, N, N]`` tensor).
-* Head dims: the kernels exist for 64 (the reference's only one) and 128.  Any other D <= 128 is
-  computed exactly by zero-padding q, k, v to 64 or 128 columns (the scores and the first D output
+* Head dims: the kernels exist for 64 (the reference's only one), 32 and 128.  Any other D <= 128
+  is computed exactly by zero-padding q, k, v to the next of these (the scores and the first D output
   columns do not change; the scale stays 1/sqrt(D)) at the price of the padding copies.
 * ``.backward()`` works.  The reference calls a ``sparse_attn_cuda.backward`` that was never
   written (:91-94); here that function exists (two HIP kernels, dQ and dK/dV, from the saved
@@ -159,10 +159,10 @@ def _check_inputs(q, k, v, mask, mask_packed=None):
 
 
 def _pad_head_dim(q, k, v):
-    """q, k, v with their head dim zero-padded to the next one the kernels have (64 or 128)."""
+    """q, k, v with their head dim zero-padded to the next one the kernels have (32, 64 or 128)."""
     D = q.shape[-1]
     assert 1 <= D <= 128, "head_dim must be at most 128"
-    Dk = 64 if D <= 64 else 128
+    Dk = 32 if D <= 32 else (64 if D <= 64 else 128)
     if D == Dk:
         return q, k, v
     pad = (0, Dk - D)
@@ -172,7 +172,7 @@ def _pad_head_dim(q, k, v):
 def sparse_attention(q, k, v, mask, mask_packed=None):
     """Masked attention with autograd support.
 
-    q, k, v: ``[B, H, N, D]`` (D = 64 or 128; other D <= 128 are zero-padded) bf16 / fp16 / fp32;  mask: bool ``[B, H, N, N]``, True = keep
+    q, k, v: ``[B, H, N, D]`` (D = 32, 64 or 128; other D <= 128 are zero-padded) bf16 / fp16 / fp32;  mask: bool ``[B, H, N, N]``, True = keep
     (a leading extent of 1 shares the mask between batch entries / heads).
     Returns a tensor of q's shape and original dtype.
 

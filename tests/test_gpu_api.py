@@ -80,8 +80,8 @@ def test_binding_rejects_bad_arguments(sa, dev):
     packed = ext.pack_mask(md)
     out = torch.empty_like(qd)
     with pytest.raises(RuntimeError, match="head_dim"):
-        ext.forward(qd[..., :32].contiguous(), kd[..., :32].contiguous(), vd[..., :32].contiguous(),
-                    packed, out[..., :32].contiguous(), None, 0.125, False)
+        ext.forward(qd[..., :48].contiguous(), kd[..., :48].contiguous(), vd[..., :48].contiguous(),
+                    packed, out[..., :48].contiguous(), None, 0.125, False)
     with pytest.raises(RuntimeError, match="Unsupported dtype"):
         ext.forward(qd.float(), kd.float(), vd.float(), packed, out.float(), None, 0.125, False)
     with pytest.raises(RuntimeError, match="lse"):

@@ -1,4 +1,4 @@
-"""GPU parity of forward and backward at head dim 128 (through the C ABI) against the fp32 oracle.
+"""GPU parity of forward and backward at head dims 32 and 128 (through the C ABI) against the fp32 oracle.
 
 The reference hard-wires head dim 64 (csrc/sparse_attention.cu:82-90, the assert at
 python/sparse_attention.py:132-134 only compares shapes), so it holds no test for this; the bar is
@@ -20,9 +20,14 @@ RTOL = {torch.float16: 1e-2, torch.bfloat16: 2e-2}
 LSE_ATOL = {torch.float16: 2e-3, torch.bfloat16: 2e-2}
 
 
-def _inputs(B, H, N, dtype, seed, keep=0.3, std=1.0):
+@pytest.fixture(params=[32, 128])
+def D(request):
+    return request.param
+
+
+def _inputs(B, H, N, dtype, seed, D, keep=0.3, std=1.0):
     g = torch.Generator().manual_seed(seed)
-    q, k, v = [(torch.randn(B, H, N, 128, generator=g) * std).to(dtype) for _ in range(3)]
+    q, k, v = [(torch.randn(B, H, N, D, generator=g) * std).to(dtype) for _ in range(3)]
     mask = torch.rand(B, H, N, N, generator=g) < keep
     return q, k, v, mask
 
@@ -49,8 +54,8 @@ def _check(out, lse, q, k, v, mask, scale=None):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("N", [1, 31, 64, 65, 128, 200, 256, 448, 512, 1000])
-def test_forward_head_dim_128(dev, dtype, N):
-    q, k, v, mask = _inputs(2, 3, N, dtype, 1000 + N)
+def test_forward(dev, dtype, N, D):
+    q, k, v, mask = _inputs(2, 3, N, dtype, 1000 + N, D)
     if N > 8:
         mask[0, 1, 5, :] = False            # a row that keeps nothing
         mask[1, 2, :, N // 2] = False       # a key that nobody keeps
@@ -59,9 +64,9 @@ def test_forward_head_dim_128(dev, dtype, N):
 
 
 @pytest.mark.parametrize("kind", ["all_true", "all_false", "diag", "block64", "causal"])
-def test_structured_masks(dev, kind):
+def test_structured_masks(dev, kind, D):
     B, H, N, dtype = 1, 2, 320, torch.float16
-    q, k, v, _ = _inputs(B, H, N, dtype, 77)
+    q, k, v, _ = _inputs(B, H, N, dtype, 77, D)
     if kind == "all_true":
         mask = torch.ones(B, H, N, N, dtype=torch.bool)
     elif kind == "all_false":
@@ -81,23 +86,23 @@ def test_structured_masks(dev, kind):
 
 
 @pytest.mark.parametrize("scale", [0.25, 1.0, 0.01, -0.5, 0.0])
-def test_scale_argument(dev, scale):
+def test_scale_argument(dev, scale, D):
     """Scales beyond 1/log2(e) take the post-multiplied exponent; at scale 1 the scores (std 11)
     leave the +-8 window of the reference point again and again."""
-    q, k, v, mask = _inputs(1, 2, 256, torch.float16, 5)
+    q, k, v, mask = _inputs(1, 2, 256, torch.float16, 5, D)
     out, lse = _run(q, k, v, mask, dev, scale=scale)
     _check(out, lse, q, k, v, mask, scale=scale)
 
 
-def test_strided_views_and_shared_mask(dev):
+def test_strided_views_and_shared_mask(dev, D):
     B, H, N, dtype = 2, 3, 200, torch.bfloat16
     g = torch.Generator().manual_seed(11)
-    qkv = torch.randn(B, N, 3, H, 128, generator=g).to(dtype)
+    qkv = torch.randn(B, N, 3, H, D, generator=g).to(dtype)
     mask = torch.rand(1, 1, N, N, generator=g) < 0.3
     qkvd = qkv.to(dev)
     q, k, v = (qkvd[:, :, i].permute(0, 2, 1, 3) for i in range(3))
     packed = _capi.pack_mask(mask.to(dev))
-    out_store = torch.full((B, N, H, 128), float("nan"), dtype=dtype, device=dev)
+    out_store = torch.full((B, N, H, D), float("nan"), dtype=dtype, device=dev)
     got = _capi.attn_fwd_strided(q, k, v, packed, out=out_store.permute(0, 2, 1, 3))
     want = _capi.attn_fwd(q.contiguous(), k.contiguous(), v.contiguous(),
                           _capi.pack_mask(mask.expand(B, H, N, N).contiguous().to(dev)))
@@ -107,13 +112,13 @@ def test_strided_views_and_shared_mask(dev):
     assert torch.allclose(got.float().cpu(), ref, atol=1e-2, rtol=2e-2)
 
 
-def test_long_sequence_and_many_heads(dev):
+def test_long_sequence_and_many_heads(dev, D):
     """N = 2112 (33 tiles, both ring slots many times over) on a few heads, and a grid of several
     rounds (B*H*tiles well beyond the 512 resident work-groups)."""
-    q, k, v, mask = _inputs(1, 2, 2112, torch.float16, 9, keep=0.1)
+    q, k, v, mask = _inputs(1, 2, 2112, torch.float16, 9, D, keep=0.1)
     out, lse = _run(q, k, v, mask, dev)
     _check(out, lse, q, k, v, mask)
-    q, k, v, mask = _inputs(8, 40, 256, torch.float16, 10, keep=0.25)
+    q, k, v, mask = _inputs(8, 40, 256, torch.float16, 10, D, keep=0.25)
     out, lse = _run(q, k, v, mask, dev)
     _check(out, lse, q, k, v, mask)
 
@@ -138,9 +143,9 @@ def _check_grads(q, k, v, do, mask, dev, scale=None):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("N", [1, 40, 64, 100, 128, 192, 333, 512])
-def test_backward_head_dim_128(dev, dtype, N):
+def test_backward(dev, dtype, N, D):
     g = torch.Generator().manual_seed(2000 + N)
-    q, k, v, do = [torch.randn(2, 2, N, 128, generator=g).to(dtype) for _ in range(4)]
+    q, k, v, do = [torch.randn(2, 2, N, D, generator=g).to(dtype) for _ in range(4)]
     mask = torch.rand(2, 2, N, N, generator=g) < 0.3
     if N > 8:
         mask[0, 1, 5, :] = False            # a row that keeps nothing: dq row 0
@@ -151,18 +156,18 @@ def test_backward_head_dim_128(dev, dtype, N):
 
 
 @pytest.mark.parametrize("scale", [0.25, 1.0, -0.5])
-def test_backward_scales(dev, scale):
+def test_backward_scales(dev, scale, D):
     g = torch.Generator().manual_seed(17)
-    q, k, v, do = [(torch.randn(1, 2, 200, 128, generator=g) * 0.7).to(torch.float16) for _ in range(4)]
+    q, k, v, do = [(torch.randn(1, 2, 200, D, generator=g) * 0.7).to(torch.float16) for _ in range(4)]
     mask = torch.rand(1, 2, 200, 200, generator=g) < 0.4
     _check_grads(q, k, v, do, mask, dev, scale=scale)
 
 
-def test_backward_strided_and_shared_mask_equals_dense(dev):
+def test_backward_strided_and_shared_mask_equals_dense(dev, D):
     B, H, N, dtype = 2, 3, 160, torch.float16
     g = torch.Generator().manual_seed(23)
-    qkv = torch.randn(B, N, 3, H, 128, generator=g).to(dtype).to(dev)
-    do = torch.randn(B, N, H, 128, generator=g).to(dtype).to(dev).permute(0, 2, 1, 3)
+    qkv = torch.randn(B, N, 3, H, D, generator=g).to(dtype).to(dev)
+    do = torch.randn(B, N, H, D, generator=g).to(dtype).to(dev).permute(0, 2, 1, 3)
     mask = (torch.rand(1, H, N, N, generator=g) < 0.3).to(dev)
     q, k, v = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
     p_small = _capi.pack_mask(mask)
@@ -178,13 +183,13 @@ def test_backward_strided_and_shared_mask_equals_dense(dev):
         assert torch.equal(g_, w_)
 
 
-def test_python_api_head_dim_128_autograd(dev):
+def test_python_api_autograd(dev, D):
     import importlib
     import sys
     importlib.import_module("python.sparse_attention")
     sa = sys.modules["python.sparse_attention"]
     g = torch.Generator().manual_seed(31)
-    q, k, v = [torch.randn(1, 2, 96, 128, generator=g).to(torch.bfloat16) for _ in range(3)]
+    q, k, v = [torch.randn(1, 2, 96, D, generator=g).to(torch.bfloat16) for _ in range(3)]
     mask = torch.rand(1, 2, 96, 96, generator=g) < 0.4
     leaves = [t.to(dev).requires_grad_(True) for t in (q, k, v)]
     out = sa.sparse_attention(*leaves, mask.to(dev))
@@ -199,10 +204,12 @@ def test_python_api_head_dim_128_autograd(dev):
         assert ((got.grad.float().cpu() - want.grad).abs() <= bound).all()
 
 
-@pytest.mark.parametrize("D", [32, 80, 96, 128])
-def test_python_api_other_head_dims(dev, D):
-    """Head dims without a kernel of their own are zero-padded by the Python layer; results and
-    gradients must be those of the operator at that head dim (scale 1/sqrt(D))."""
+@pytest.mark.parametrize("Dx", [8, 24, 40, 80, 96, 120])
+def test_python_api_other_head_dims(dev, Dx):
+    """Head dims without a kernel of their own are zero-padded by the Python layer to the next of
+    32, 64, 128; results and gradients must be those of the operator at that head dim (scale
+    1/sqrt(D))."""
+    D = Dx
     import importlib
     import sys
     importlib.import_module("python.sparse_attention")

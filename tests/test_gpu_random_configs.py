@@ -55,7 +55,7 @@ def _mask(rng, g, Bm, Hm, N):
 def test_random_configuration(dev, seed):
     rng = random.Random(seed)
     g = torch.Generator().manual_seed(seed)
-    D = rng.choice([64, 128])
+    D = rng.choice([32, 64, 128])
     dtype = rng.choice([torch.float16, torch.bfloat16])
     B, H = rng.choice([(1, 1), (1, 3), (2, 2), (3, 1)])
     N = rng.choice([1, 7, 32, 63, 64, 65, 100, 127, 128, 129, 191, 192, 250, 320, 401])

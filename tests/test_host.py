@@ -41,7 +41,7 @@ def test_argument_validation_needs_no_gpu(capi):
         a = dict(ok_args, **kw)
         return f(q, k, v, mp, out, lse, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
 
-    assert call(D=32) == _capi.SMA_ERR_HEAD_DIM
+    assert call(D=16) == _capi.SMA_ERR_HEAD_DIM
     assert call(D=96) == _capi.SMA_ERR_HEAD_DIM
     assert call(D=256) == _capi.SMA_ERR_HEAD_DIM
     assert call(dtype=2) == _capi.SMA_ERR_DTYPE
@@ -53,6 +53,7 @@ def test_argument_validation_needs_no_gpu(capi):
     assert call(q=ctypes.c_void_p(0x1002)) == _capi.SMA_ERR_ALIGNMENT
     assert call(B=0) == _capi.SMA_OK and call(N=0) == _capi.SMA_OK          # empty problem: nothing to do
     assert call(B=1 << 20, H=1 << 12, N=64) == _capi.SMA_ERR_BAD_SHAPE      # index range
+    assert call(B=1, H=1, N=200000) == _capi.SMA_ERR_BAD_SHAPE              # packed mask of one (b,h) beyond 4 GiB
 
     # strided entry point: the descriptor is checked before anything is launched
     fs = capi.sma_attn_fwd_strided
