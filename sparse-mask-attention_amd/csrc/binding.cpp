@@ -36,6 +36,7 @@ void check_status(int st, const char *what)
 // (PyTorch leaves their strides arbitrary).
 sma_tensor rows_of(const torch::Tensor &t, const char *name)
 {
+    if (t.numel() == 0) return sma_tensor{t.data_ptr(), 0, 0, 0};     // nothing will be read or written
     TORCH_CHECK(t.stride(3) == 1 || t.size(3) == 1, name, ": the last dimension must be contiguous");
     sma_tensor d;
     d.data = t.data_ptr();

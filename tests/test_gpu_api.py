@@ -244,3 +244,20 @@ def test_layouts_the_kernels_cannot_address_are_copied(sa, dev):
         assert torch.equal(sa.sparse_attention_func(view, k.to(dev), v.to(dev), md), want)
     qt = q.to(dev).transpose(2, 3).contiguous().transpose(2, 3)
     assert torch.equal(sa.sparse_attention_func(qt, k.to(dev), v.to(dev), md), want)
+
+
+@pytest.mark.parametrize("shape", [(0, 2, 16), (2, 0, 16), (1, 1, 0)])
+def test_empty_problems_are_no_ops(sa, dev, shape):
+    """Zero batch entries, heads or sequence length: nothing is launched, shapes come back right,
+    and autograd still returns (empty) gradients."""
+    B, H, N = shape
+    q, k, v = [torch.zeros(B, H, N, 64, dtype=torch.float16, device=dev, requires_grad=True) for _ in range(3)]
+    mask = torch.zeros(B, H, N, N, dtype=torch.bool, device=dev)
+    packed = sa.pack_mask(mask)
+    assert packed.shape == (B, H, N, (N + 31) // 32) and packed.dtype == torch.int32
+    out = sa.sparse_attention(q, k, v, mask)
+    assert out.shape == (B, H, N, 64)
+    out.sum().backward()
+    assert q.grad.shape == q.shape and k.grad.shape == k.shape and v.grad.shape == v.shape
+    assert sa.sparse_attention_func(q.detach(), k.detach(), v.detach(), mask).shape == (B, H, N, 64)
+    torch.cuda.synchronize()
