@@ -261,3 +261,15 @@ def test_empty_problems_are_no_ops(sa, dev, shape):
     assert q.grad.shape == q.shape and k.grad.shape == k.shape and v.grad.shape == v.shape
     assert sa.sparse_attention_func(q.detach(), k.detach(), v.detach(), mask).shape == (B, H, N, 64)
     torch.cuda.synchronize()
+
+
+def test_backward_from_an_expanded_gradient(sa, dev):
+    """out.sum().backward() hands the autograd function a gradient whose strides are all zero."""
+    q, k, v, mask = _inputs(1, 2, 80, torch.float16, 12, keep=0.4)
+    leaves = [t.to(dev).requires_grad_(True) for t in (q, k, v)]
+    sa.sparse_attention(*leaves, mask.to(dev)).sum().backward()
+    refs = [t.float().requires_grad_(True) for t in (q, k, v)]
+    O.sparse_attention_ref(*refs, mask).sum().backward()
+    for got, want in zip(leaves, refs):
+        bound = 1e-4 + 1e-2 * want.grad.abs().max() + 1e-2 * want.grad.abs()
+        assert ((got.grad.float().cpu() - want.grad).abs() <= bound).all()
