@@ -430,21 +430,24 @@ __global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD)
     // ---- epilogue ----
     // out = O / l.  The accumulator layout gives a lane 8-byte pieces of one row; written as they
     // are, a store instruction would touch 32 different 128-byte rows.  Each wave therefore
-    // transposes its 32 x 64 block (one per column half) through 4 KiB of LDS (K/V stage 0, free
-    // after a barrier) and stores whole 128-byte pieces of rows, non-temporally: the output is not
-    // read again here and should not displace K, V and the mask.
+    // transposes its 32 x 64 block (one per column half) through 4 KiB of LDS and stores whole
+    // 128-byte pieces of rows, non-temporally: the output is not read again here and should not
+    // displace K, V and the mask.  The LDS used is the stage that tile T would have gone to: its
+    // last occupant was tile T - NSTAGE, which every wave had finished before the barrier of the
+    // last iteration, and no copy into it is in flight, so no further barrier is needed and a wave
+    // that is done early stores early.
     const float l_tot = xhalf_sum(l_run);
     const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
-    __syncthreads();              // every wave is done reading the K/V stages
     {
         const int row0 = qt * BM + wave * 32;
         uint16_t *ob = slab(a.out, bi, hi) + (size_t)row0 * o_sn;
+        const uint32_t ebase = lds0 + (uint32_t)(T % NSTAGE) * STAGE_BYTES + wave * 4096;
         if constexpr (HDIM == 32) {
-            store_block<BF16, 32>(oacc[0], oacc[0], inv, lds0 + wave * 4096, ob, (int)o_sn, row0, N, lane);
+            store_block<BF16, 32>(oacc[0], oacc[0], inv, ebase, ob, (int)o_sn, row0, N, lane);
         } else {
 #pragma unroll
             for (int half = 0; half < NH; ++half)
-                store_block<BF16>(oacc[2 * half], oacc[2 * half + 1], inv, lds0 + wave * 4096 + half * 16384,
+                store_block<BF16>(oacc[2 * half], oacc[2 * half + 1], inv, ebase + half * 16384,
                                   ob + half * HD, (int)o_sn, row0, N, lane);
         }
     }
