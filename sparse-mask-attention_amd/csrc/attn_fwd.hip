@@ -38,6 +38,7 @@
 //   head dim    = the description above is for 64.  128 runs the same code on two column halves of
 //                 64 (see Cfg below): twice the MFMAs per tile for the same softmax work, a ring of
 //                 two stages and two work-groups per CU.  32 uses half of every tile row.
+#include <atomic>
 #include <type_traits>
 
 #include "attn_common.h"
@@ -465,14 +466,13 @@ __global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD)
 // Number of compute units of the current device (cached per device ordinal).
 static int compute_units()
 {
-    static int cached[64];
+    static std::atomic<int> cached[64];      // 0 = not asked yet; threads may race to store the same value
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 0;
-    if (cached[dev] == 0) {
-        int n = 0;
-        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess) cached[dev] = n;
-    }
-    return cached[dev];
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0 && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess)
+        cached[dev].store(n, std::memory_order_relaxed);
+    return n;
 }
 
 hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)

@@ -27,7 +27,8 @@ What differs from the reference, on purpose:
   if they were contiguous; anything else is copied with ``.contiguous()`` first.
 * ``mask`` may be ``[1, 1, N, N]``, ``[B, 1, N, N]`` or ``[1, H, N, N]``: it is packed once at that
   size and shared between batch entries / heads by the kernels (the reference needs the expanded
-  ``[B, H, N, N]`` tensor).
+  ``[B, H, N, N]`` tensor).  A mask passed as an ``expand``-ed view is recognised by its zero
+  strides and treated the same way.
 * Head dims: the kernels exist for 64 (the reference's only one), 32 and 128.  Any other D <= 128
   is computed exactly by zero-padding q, k, v to the next of these (the scores and the first D output
   columns do not change; the scale stays 1/sqrt(D)) at the price of the padding copies.
@@ -158,6 +159,16 @@ def _check_inputs(q, k, v, mask, mask_packed=None):
         "mask must be [B or 1, H or 1, N, N]"
 
 
+def _pack_shared(mask: torch.Tensor) -> torch.Tensor:
+    """pack_mask of the mask with its expanded (stride 0) batch / head extents taken back to 1: a
+    mask given as ``m.expand(B, H, N, N)`` is packed once and shared, not B*H times."""
+    if mask.size(0) > 1 and mask.stride(0) == 0:
+        mask = mask[:1]
+    if mask.size(1) > 1 and mask.stride(1) == 0:
+        mask = mask[:, :1]
+    return pack_mask(mask)
+
+
 def _pad_head_dim(q, k, v):
     """q, k, v with their head dim zero-padded to the next one the kernels have (32, 64 or 128)."""
     D = q.shape[-1]
@@ -190,7 +201,7 @@ def sparse_attention(q, k, v, mask, mask_packed=None):
         q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
 
     if mask_packed is None:
-        mask_packed = pack_mask(mask)
+        mask_packed = _pack_shared(mask)
     q, k, v = _pad_head_dim(q, k, v)              # differentiable: the gradients are sliced back
     out = SparseAttentionFunction.apply(q, k, v, mask_packed, mask, scale, N)[..., :D]
 
@@ -214,7 +225,7 @@ def sparse_attention_func(q, k, v, mask, mask_packed=None):
         q, k, v = _pad_head_dim(q, k, v)
         q, k, v = _rows(q), _rows(k), _rows(v)
         if mask_packed is None:
-            mask_packed = pack_mask(mask)
+            mask_packed = _pack_shared(mask)
         out = torch.empty_like(q)
         sparse_attn_cuda.forward(q, k, v, mask_packed, out, None, scale, False)
         out = out[..., :D]

@@ -273,3 +273,20 @@ def test_backward_from_an_expanded_gradient(sa, dev):
     for got, want in zip(leaves, refs):
         bound = 1e-4 + 1e-2 * want.grad.abs().max() + 1e-2 * want.grad.abs()
         assert ((got.grad.float().cpu() - want.grad).abs() <= bound).all()
+
+
+def test_expanded_mask_is_packed_once(sa, dev, monkeypatch):
+    """mask.expand(B, H, N, N) (zero strides) must reach the packer with the extents it really has."""
+    B, H, N = 3, 4, 96
+    q, k, v, _ = _inputs(B, H, N, torch.float16, 14)
+    g = torch.Generator().manual_seed(15)
+    small = (torch.rand(1, 1, N, N, generator=g) < 0.3).to(dev)
+    seen = []
+    real = sa.pack_mask
+    monkeypatch.setattr(sa, "pack_mask", lambda m: (seen.append(tuple(m.shape)), real(m))[1])
+    out = sa.sparse_attention_func(q.to(dev), k.to(dev), v.to(dev), small.expand(B, H, N, N))
+    out_h = sa.sparse_attention_func(q.to(dev), k.to(dev), v.to(dev), small.expand(1, H, N, N).contiguous().expand(B, H, N, N))
+    assert seen == [(1, 1, N, N), (1, H, N, N)]
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), small.cpu().expand(B, H, N, N))
+    assert torch.allclose(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+    assert torch.equal(out, out_h)
