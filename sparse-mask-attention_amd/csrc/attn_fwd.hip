@@ -6,7 +6,7 @@
 //
 // Work decomposition
 //   work-group  = 4 wavefronts = 128 query rows of one (b,h); it walks the keys in tiles of 64.
-//                 Three work-groups fit a CU (<= 168 VGPRs, ~52 KB LDS each): one wavefront of
+//                 Three work-groups fit a CU (<= 168 VGPRs, ~34 KB LDS each): one wavefront of
 //                 each per SIMD, so that the softmax VALU work of one overlaps the MFMAs of another.
 //   wavefront   = 32 query rows.  It computes S^T = K_tile (64x64) * Q^T (64x32) with
 //                 v_mfma_f32_32x32x16, so every lane owns ONE query row (lane % 32) and 32 of the
@@ -14,14 +14,14 @@
 //                 exchange between lane l and lane l+32 (v_permlane32_swap).  P^T is already in
 //                 the B-operand layout of O^T += V^T * P^T: probabilities never leave registers.
 //   K/V tiles   = copied global -> LDS by global_load_lds_dwordx4 (no VGPR staging) into a ring of
-//                 three stages, two tiles ahead of the one being computed.  Rows are 128 B; the
+//                 two stages, one tile ahead of the one being computed.  Rows are 128 B; the
 //                 16-byte chunks of a row are XOR-swizzled (the permutation is applied to the
 //                 global address of each lane; the LDS side of such a load is always linear) so
 //                 that K's ds_read_b128 (32 consecutive rows, same column) and V's
 //                 ds_read_b64_tr_b16 (transposing read, 8 consecutive rows x 64 B) are free of
 //                 bank conflicts on the 64-bank LDS.
 //   mask        = each wavefront copies the two packed words per query row of a tile into LDS with
-//                 one global_load_lds_dword, two tiles ahead.  A lane reads the two words of its
+//                 one global_load_lds_dword, one tile ahead.  A lane reads the two words of its
 //                 row; each nibble selects one of 16 rows of a small LDS table of four floats that
 //                 are 0 (keep) or -inf (drop); one ds_read_b128 of that row initialises four
 //                 accumulator registers of the QK^T MFMA chain.  Masking costs no VALU work per score.
@@ -57,13 +57,13 @@ constexpr float WINDOW_LOG2 = 8.0f;
 // read patterns:
 //   128  two column halves (NH = 2): K and V tiles are kept in LDS as two 64-column tiles each, the
 //        QK^T chain runs over both halves of K and q, and P multiplies each half of V into its own
-//        pair of accumulators.  A stage is twice as large, so the ring has two stages (copies one
-//        tile ahead) and two work-groups share a CU.
+//        pair of accumulators.  A stage is twice as large (32 KiB) and the kernel needs about 224
+//        registers, so two work-groups share a CU.
 //   32   half a tile: the copies fill the upper half of every LDS row with a second copy of the
 //        lower half (global chunk index & 3), which is never read; the QK^T chain has two steps
 //        instead of four and P multiplies one 32-column block of V.
 template <int NH> struct Cfg {
-    static constexpr int NSTAGE = NH == 1 ? 3 : 2;
+    static constexpr int NSTAGE = 2;                                // ring of two stages: copies run one tile ahead
     static constexpr int WAVES_PER_SIMD = NH == 1 ? 3 : 2;
     static constexpr int COPIES = 1 + 4 * NH;                       // async copies per wave and tile
     // LDS map (bytes)
@@ -219,9 +219,8 @@ __global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD)
     const uint32_t nib_shift = 4u - 4u * hh;
 
     // ================================ prologue: one memory round trip ================================
-    // Requested at once, oldest first: q (this wave's 32 rows, staged through the last K/V stage,
-    // which the prologue leaves unused, K-swizzled), then the mask words and K/V of the first
-    // NSTAGE - 1 tiles.
+    // Requested at once, oldest first: q (this wave's 32 rows, staged through the second K/V stage,
+    // which the prologue leaves unused, K-swizzled), then the mask words and K/V of tile 0.
     const int qrow = qt * BM + wave * 32 + l32;
     {
         const int qbase = qt * BM + wave * 32 < N ? qt * BM + wave * 32 : N - 1;   // wave-uniform
@@ -246,12 +245,7 @@ __global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
     const bool even_progress = NH == 1 && (int)blockIdx.x >= a.tail_start;   // three work-groups per CU
     if (even_progress && T >= 4) __builtin_amdgcn_s_setprio(3);
-    if constexpr (NSTAGE == 3) {
-        if (T > 1) { issue_mask(1, integral_constant<int, 1>{}); issue_kv(1, integral_constant<int, 1>{}); }
-        if (T > 1) wait_vmcnt<2 * C::COPIES>(); else wait_vmcnt<C::COPIES>();       // q has landed
-    } else {
-        wait_vmcnt<C::COPIES>();
-    }
+    wait_vmcnt<C::COPIES>();          // q has landed; the copies of tile 0 may still be in flight
     // ---- Q^T as MFMA B operands, scaled by scale*log2(e)/post_mul:
     //      lane holds query row l32, d = 16*s + 8*hh .. +7
     u32x4 qf[KS];
@@ -390,16 +384,19 @@ __global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD)
     };
 
     // ================================ main loop ================================
-    // Tile t uses stage and mask slot t % NSTAGE; the loop is unrolled by NSTAGE so that these are
-    // constants.  In iteration t:
-    //   wait for the copies of tile t  ->  barrier  ->  request the copies of tile t + NSTAGE - 1
-    //   (mask words, then K/V)  ->  compute, unless this wave's 32 x 64 block of mask bits is empty.
+    // Tile t uses stage and mask slot t % 2; the loop is unrolled by 2 so that these are constants.
+    // In iteration t:
+    //   wait for the copies of tile t  ->  barrier  ->  request the copies of tile t + 1 (mask
+    //   words, then K/V) into the stage the barrier has freed  ->  compute, unless this wave's
+    //   32 x 64 block of mask bits is empty.
+    // (A ring of three stages, copies two tiles ahead, measured the same to 2 % slower on every
+    // workload and costs 18 KB more LDS.)
     // Every tile is copied: exchanging per-tile "is any of the 128 rows live" flags between the
     // waves (tried: through LDS two tiles ahead, and as a bit map built up front from the mask
     // rows) cost more than the copies it saved, on block-structured masks too.
     auto iteration = [&](const int t, auto slot_c) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
-        constexpr int SLOT2 = (SLOT + NSTAGE - 1) % NSTAGE;       // the stage freed by the barrier below
+        constexpr int SLOT2 = SLOT ^ 1;       // the stage freed by the barrier below
         if (even_progress) {
             // The hardware serves the oldest wave first, so of three co-resident work-groups one
             // finishes early and the last runs alone, at a worse rate than three together.  When
@@ -408,23 +405,19 @@ __global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD)
             else if (t == T / 2) __builtin_amdgcn_s_setprio(1);
             else if (t == (3 * T) / 4) __builtin_amdgcn_s_setprio(0);
         }
-        // copies complete in issue order; only those of the tiles requested after tile t may stay in flight
-        if (NSTAGE == 3 && t + 1 < T) wait_vmcnt<C::COPIES>(); else wait_vmcnt<0>();
+        wait_vmcnt<0>();          // the copies of tile t (the only ones in flight) have landed
         if (ragged && t == T - 1) zero_tail_rows(t, SLOT);
         __syncthreads();          // tile t landed for every wave; the stage of tile t - 1 is free
         const u32x2 w2 = mask_words(t, SLOT);
-        if (t + NSTAGE - 1 < T) {
-            issue_mask(t + NSTAGE - 1, integral_constant<int, SLOT2>{});
-            issue_kv(t + NSTAGE - 1, integral_constant<int, SLOT2>{});
+        if (t + 1 < T) {
+            issue_mask(t + 1, integral_constant<int, SLOT2>{});
+            issue_kv(t + 1, integral_constant<int, SLOT2>{});
         }
         compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
     };
-    for (int t = 0; t < T; t += NSTAGE) {
+    for (int t = 0; t < T; t += 2) {
         iteration(t, integral_constant<int, 0>{});
         if (t + 1 < T) iteration(t + 1, integral_constant<int, 1>{});
-        if constexpr (NSTAGE == 3) {
-            if (t + 2 < T) iteration(t + 2, integral_constant<int, 2>{});
-        }
     }
     wait_vmcnt<0>();              // no copy may outlive the work-group's LDS allocation
 
@@ -434,8 +427,8 @@ __global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD)
     // transposes its 32 x 64 block (one per column half) through 4 KiB of LDS and stores whole
     // 128-byte pieces of rows, non-temporally: the output is not read again here and should not
     // displace K, V and the mask.  The LDS used is the stage that tile T would have gone to: its
-    // last occupant was tile T - NSTAGE, which every wave had finished before the barrier of the
-    // last iteration, and no copy into it is in flight, so no further barrier is needed and a wave
+    // last occupant was tile T - 2, which every wave had finished before the barrier of the last
+    // iteration, and no copy into it is in flight, so no further barrier is needed and a wave
     // that is done early stores early.
     const float l_tot = xhalf_sum(l_run);
     const float inv = (l_tot > 0.f) ? 1.0f / l_tot : 0.f;
