@@ -124,6 +124,27 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
                          const sma_tensor *out, float *lse, int B, int H, int N, int D, float scale,
                          int dtype, void *stream);
 
+/* sma_pack_mask and sma_attn_fwd in one launch, for a mask that is used once: the kernel reads the
+ * boolean bytes themselves and forms the packed words of each 64-key tile on the fly, so the packing
+ * pass, its launch and the round trip of the words through memory disappear.
+ *
+ *   q, k, v, out    contiguous [B,H,N,D], D = 32 or 64; N must be a multiple of 64
+ *   mask            uint8 [Bm,Hm,N,N] with Bm in {1,B}, Hm in {1,H}, rows contiguous, 16-byte aligned;
+ *                   every byte must be 0 or 1 (torch.bool storage; unlike sma_pack_mask, other
+ *                   non-zero values are not accepted); mask_stride_b / mask_stride_h in BYTES,
+ *                   multiples of 16, 0 = shared between batch entries / heads
+ *   lse             NULL or float [B,H,N]
+ *
+ * Anything outside these limits returns an error code and is served by sma_pack_mask followed by
+ * sma_attn_fwd (or its strided form), which give the same results.
+ *
+ * Replaces: the pair of launches the reference's forward makes for every call,
+ *           python/sparse_attention.py:146 + :171 (pack_mask, then forward), run.py:151-154.
+ */
+int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const uint8_t *mask,
+                           int64_t mask_stride_b, int64_t mask_stride_h, void *out, float *lse,
+                           int B, int H, int N, int D, float scale, int dtype, void *stream);
+
 /* sma_attn_bwd for strided dout, q, k, v, out, dq, dk, dv and a shared mask (see
  * sma_attn_fwd_strided); lse and delta_ws are contiguous float [B,H,N].
  */

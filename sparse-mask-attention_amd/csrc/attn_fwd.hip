@@ -62,15 +62,22 @@ constexpr float WINDOW_LOG2 = 8.0f;
 //   32   half a tile: the copies fill the upper half of every LDS row with a second copy of the
 //        lower half (global chunk index & 3), which is never read; the QK^T chain has two steps
 //        instead of four and P multiplies one 32-column block of V.
-template <int NH> struct Cfg {
+//
+// BYTEMASK: the mask arrives as the caller's boolean bytes (one per score, 0 or 1) instead of packed
+// words.  Each wavefront copies the 32 x 64 bytes of a tile for its rows into LDS and turns them
+// into the two words per row itself (eight dot products with the weights 1, 2, 4 .. 128 per lane
+// and one exchange between the lane halves): the separate packing pass, its launch and the
+// round trip of the words through memory disappear for a mask that is used once.
+template <int NH, bool BYTEMASK> struct Cfg {
     static constexpr int NSTAGE = 2;                                // ring of two stages: copies run one tile ahead
-    static constexpr int WAVES_PER_SIMD = NH == 1 ? 3 : 2;
-    static constexpr int COPIES = 1 + 4 * NH;                       // async copies per wave and tile
+    static constexpr int MASK_COPIES = BYTEMASK ? 2 : 1;
+    static constexpr int COPIES = MASK_COPIES + 4 * NH;             // async copies per wave and tile
     // LDS map (bytes)
     static constexpr int STAGE_BYTES = 2 * NH * TILE_BYTES;         // K halves, then V halves
     static constexpr int OFF_V = NH * TILE_BYTES;                   // V inside a stage
-    static constexpr int OFF_MASK = NSTAGE * STAGE_BYTES;           // NSTAGE slots x 4 waves x 64 words
-    static constexpr int OFF_LUT = OFF_MASK + NSTAGE * 1024;        // 16 x 16 B
+    static constexpr int OFF_MASK = NSTAGE * STAGE_BYTES;           // NSTAGE slots x 4 waves x (64 words | 2 KiB of bytes)
+    static constexpr int MASK_SLOT = BYTEMASK ? 8192 : 1024;
+    static constexpr int OFF_LUT = OFF_MASK + NSTAGE * MASK_SLOT;   // 16 x 16 B
     static constexpr int LDS_BYTES = OFF_LUT + 256;
 };
 
@@ -79,16 +86,17 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_
 // PACKED_ROWS: the rows of q, k, v and out follow each other without gaps (row stride 64), as in
 // contiguous tensors; the strides between heads and batch entries stay free.  A row stride known
 // at compile time measured 0.25 us less fixed cost per launch than the same value read at run time.
-template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int HDIM>
-__global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD) void attn_fwd_kernel(const AttnArgs a)
+template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int HDIM, bool BYTEMASK = false>
+__global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel(const AttnArgs a)
 {
     using E = Elem<BF16>;
     constexpr int NH = HDIM == 128 ? 2 : 1;       // 64-column tiles per matrix
     constexpr int KS = HDIM / 16;                 // MFMA steps of the QK^T chain
     constexpr int OB = HDIM / 32;                 // 32-column accumulator blocks of O
     constexpr int CHM = HDIM == 32 ? 3 : 7;       // 16-byte chunks per global row, minus one
-    using C = Cfg<NH>;
+    using C = Cfg<NH, BYTEMASK>;
     constexpr int NSTAGE = C::NSTAGE, STAGE_BYTES = C::STAGE_BYTES, OFF_MASK = C::OFF_MASK, OFF_LUT = C::OFF_LUT;
+    constexpr int MASK_SLOT = C::MASK_SLOT;
     constexpr int D = HDIM;
     __shared__ __attribute__((aligned(1024))) unsigned char smem[C::LDS_BYTES];
     const uint32_t lds0 = (uint32_t)(uintptr_t)(LDS_PTR(unsigned char))smem;
@@ -110,24 +118,66 @@ __global__ __launch_bounds__(NTHREADS, Cfg<HDIM == 128 ? 2 : 1>::WAVES_PER_SIMD)
     const uint16_t *qb = slab(a.q, bi, hi);
     const uint16_t *kb = slab(a.k, bi, hi);
     const uint16_t *vb = slab(a.v, bi, hi);
-    const uint32_t *mb = slab(a.mask, bi, hi);
+    // packed: words, strides in words; BYTEMASK: bytes, strides in bytes
+    const uint32_t *mb = BYTEMASK ? reinterpret_cast<const uint32_t *>(reinterpret_cast<const uint8_t *>(a.mask.p) +
+                                                                       bi * a.mask.sb + hi * a.mask.sh)
+                                  : slab(a.mask, bi, hi);
     const uint32_t q_sn = PACKED_ROWS ? D : a.q.sn, k_sn = PACKED_ROWS ? D : a.k.sn;       // row strides, elements
     const uint32_t v_sn = PACKED_ROWS ? D : a.v.sn, o_sn = PACKED_ROWS ? D : a.out.sn;
     const uint32_t q_rb = 2u * q_sn, k_rb = 2u * k_sn, v_rb = 2u * v_sn;                   // row pitch, bytes
 
     // ---- mask words: wave-private async copies, slot = tile % NSTAGE, lane i -> (row i/2, word i%2) ----
-    const int mrow = qt * BM + wave * 32 + (lane >> 1);
-    const uint32_t m_voff = (uint32_t)(((size_t)(mrow < N ? mrow : N - 1) * nw + (lane & 1)) * 4);
-    const uint32_t mask_dst = lds0 + wave * 256;
+    // BYTEMASK (N % 64 == 0): the wave's 32 x 64 bytes of a tile as two copies of 16 rows; lane i
+    // fills (row 16j + i/4, position i%4) with the global 16-byte chunk position ^ ((row >> 2) & 3),
+    // which makes the reads below (lane = row, two chunks each) free of bank conflicts.
+    const int mrow = BYTEMASK ? 0 : qt * BM + wave * 32 + (lane >> 1);
+    const uint32_t m_voff = BYTEMASK ? 0u : (uint32_t)(((size_t)(mrow < N ? mrow : N - 1) * nw + (lane & 1)) * 4);
+    uint32_t mb_voff[2] = {0u, 0u};
+    if constexpr (BYTEMASK) {
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int row = 16 * j + (lane >> 2);
+            const int grow = qt * BM + wave * 32 + row;
+            mb_voff[j] = (uint32_t)(grow < N ? grow : N - 1) * (uint32_t)N + (uint32_t)(((lane & 3) ^ ((row >> 2) & 3)) << 4);
+        }
+    }
+    const uint32_t mask_dst = lds0 + wave * (BYTEMASK ? 2048 : 256);
     auto issue_mask = [&](int x, auto slot_c) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
-        uint32_t voff = m_voff;
-        if (2 * x + 1 >= nw) voff -= (lane & 1) * 4;           // odd word count: re-read the last word
-        async_copy_b32_at<OFF_MASK + SLOT * 1024>(mask_dst, mb + 2 * x, voff);
+        if constexpr (BYTEMASK) {
+            const uint8_t *src = reinterpret_cast<const uint8_t *>(mb) + (size_t)x * BN;
+            async_copy_b128_at<OFF_MASK + SLOT * MASK_SLOT>(mask_dst, src, mb_voff[0]);
+            async_copy_b128_at<OFF_MASK + SLOT * MASK_SLOT + 1024>(mask_dst, src, mb_voff[1]);
+        } else {
+            uint32_t voff = m_voff;
+            if (2 * x + 1 >= nw) voff -= (lane & 1) * 4;           // odd word count: re-read the last word
+            async_copy_b32_at<OFF_MASK + SLOT * MASK_SLOT>(mask_dst, mb + 2 * x, voff);
+        }
     };
-    const uint32_t maddr = lds0 + OFF_MASK + wave * 256 + l32 * 8;
+    const uint32_t maddr = BYTEMASK ? lds0 + OFF_MASK + wave * 2048 + l32 * 64 : lds0 + OFF_MASK + wave * 256 + l32 * 8;
+    const int msw = (l32 >> 2) & 3;
     auto mask_words = [&](int x, int slot) __attribute__((always_inline)) -> u32x2 {
-        u32x2 w = lds_read_b64(maddr + slot * 1024);
+        u32x2 w;
+        if constexpr (BYTEMASK) {
+            // this lane: the 32 bytes of row l32 for keys 32hh .. 32hh+31 -> one word
+            const u32x4 d0 = lds_read_b128(maddr + slot * MASK_SLOT + (((2 * hh) ^ msw) << 4));
+            const u32x4 d1 = lds_read_b128(maddr + slot * MASK_SLOT + (((2 * hh + 1) ^ msw) << 4));
+            uint32_t b0 = __builtin_amdgcn_udot4(d0.x, 0x08040201u, 0u, false);
+            uint32_t b1 = __builtin_amdgcn_udot4(d0.z, 0x08040201u, 0u, false);
+            uint32_t b2 = __builtin_amdgcn_udot4(d1.x, 0x08040201u, 0u, false);
+            uint32_t b3 = __builtin_amdgcn_udot4(d1.z, 0x08040201u, 0u, false);
+            b0 = __builtin_amdgcn_udot4(d0.y, 0x80402010u, b0, false);
+            b1 = __builtin_amdgcn_udot4(d0.w, 0x80402010u, b1, false);
+            b2 = __builtin_amdgcn_udot4(d1.y, 0x80402010u, b2, false);
+            b3 = __builtin_amdgcn_udot4(d1.w, 0x80402010u, b3, false);
+            const uint32_t mine = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            // lanes < 32 hold the word of keys 0..31, lanes >= 32 that of keys 32..63: both to both
+            const auto r = __builtin_amdgcn_permlane32_swap(mine, mine, false, false);
+            w.x = (uint32_t)r[0];
+            w.y = (uint32_t)r[1];
+        } else {
+            w = lds_read_b64(maddr + slot * MASK_SLOT);
+        }
         const bool last = (x == T - 1);
         w.x &= last ? a.last_mask0 : 0xffffffffu;
         w.y &= last ? a.last_mask1 : 0xffffffffu;
@@ -498,8 +548,20 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     case 6: kernel = attn_fwd_kernel<true, true, false, HDIM>; break;                  \
     default: kernel = attn_fwd_kernel<true, true, true, HDIM>; break;                  \
     }
-    if (D == 32) { SMA_FWD_VARIANTS(32) } else if (D == 64) { SMA_FWD_VARIANTS(64) } else { SMA_FWD_VARIANTS(128) }
+#define SMA_FWD_BYTEMASK_VARIANTS(HDIM)                                                 \
+    switch (variant >> 1) {                                                            \
+    case 0: kernel = attn_fwd_kernel<false, false, true, HDIM, true>; break;           \
+    case 1: kernel = attn_fwd_kernel<false, true, true, HDIM, true>; break;            \
+    case 2: kernel = attn_fwd_kernel<true, false, true, HDIM, true>; break;            \
+    default: kernel = attn_fwd_kernel<true, true, true, HDIM, true>; break;            \
+    }
+    if (a.byte_mask) {
+        // built for contiguous rows and head dims 32 and 64 only (checked by the C-ABI layer)
+        if (!packed || D == 2 * HD || (a.N & (BN - 1)) != 0) return hipErrorInvalidValue;
+        if (D == 32) { SMA_FWD_BYTEMASK_VARIANTS(32) } else { SMA_FWD_BYTEMASK_VARIANTS(64) }
+    } else if (D == 32) { SMA_FWD_VARIANTS(32) } else if (D == 64) { SMA_FWD_VARIANTS(64) } else { SMA_FWD_VARIANTS(128) }
 #undef SMA_FWD_VARIANTS
+#undef SMA_FWD_BYTEMASK_VARIANTS
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, a);
     return hipGetLastError();
 }

@@ -8,6 +8,9 @@
 //   pack_mask(mask) -> int32 Tensor [B, H, N, ceil(N/32)]
 //   backward(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, scale) -> None   (called by the
 //       reference's Python API, python/sparse_attention.py:91-94, but absent from its binding)
+//   forward_bool_mask(q, k, v, mask, out, lse, scale, is_training) -> None   (not in the reference:
+//       `forward` with the boolean mask itself in place of the packed one, one launch instead of
+//       pack_mask + forward; `bool_mask_supported(q, k, v, mask)` says whether it applies)
 //
 // Differences, all on the safe side: `lse` may be None (the reference's own inference wrapper
 // passes None, python/sparse_attention.py:170-171); every tensor argument is checked (device,
@@ -101,6 +104,61 @@ void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor
     check_status(st, "sma_attn_fwd_strided");
 }
 
+// Limits of sma_attn_fwd_bool_mask, so that callers can choose between it and pack_mask + forward
+// without provoking an error: contiguous q, k, v, head dim 32 or 64, N a multiple of 64, a
+// contiguous bool mask [1|B, 1|H, N, N] whose storage is 16-byte aligned.
+bool bool_mask_supported(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,
+                         const torch::Tensor &mask)
+{
+    if (!q.is_cuda() || q.dim() != 4 || mask.dim() != 4) return false;
+    const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
+    if (!(D == 32 || D == 64) || N % 64 != 0 || N == 0 || N * N >= (int64_t(1) << 31)) return false;
+    if (!q.is_contiguous() || !k.is_contiguous() || !v.is_contiguous()) return false;
+    if (mask.scalar_type() != at::kBool || !mask.is_contiguous() || mask.device() != q.device()) return false;
+    if (!((mask.size(0) == B || mask.size(0) == 1) && (mask.size(1) == H || mask.size(1) == 1) &&
+          mask.size(2) == N && mask.size(3) == N))
+        return false;
+    return reinterpret_cast<uintptr_t>(mask.data_ptr()) % 16 == 0;
+}
+
+void forward_bool_mask(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,
+                       const torch::Tensor &mask, torch::Tensor out,
+                       const c10::optional<torch::Tensor> &lse, double scale, bool is_training)
+{
+    TORCH_CHECK(q.is_cuda(), "q must be a GPU tensor");
+    TORCH_CHECK(q.dim() == 4, "q must be 4D [B, H, N, D]");
+    const auto dt = q.scalar_type();
+    TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "Unsupported dtype, need BF16 or FP16");
+    TORCH_CHECK(bool_mask_supported(q, k, v, mask),
+                "forward_bool_mask needs contiguous q, k, v with head_dim 32 or 64, N a multiple of 64 and a "
+                "contiguous bool mask [B or 1, H or 1, N, N]; use pack_mask + forward otherwise");
+    const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
+    for (const torch::Tensor *t : {&k, &v, static_cast<const torch::Tensor *>(&out)}) {
+        TORCH_CHECK(t->device() == q.device(), "q, k, v, out must be on the same device");
+        TORCH_CHECK(t->scalar_type() == dt, "q, k, v, out must have the same dtype");
+        TORCH_CHECK(t->sizes() == q.sizes(), "q, k, v, out must have the same shape");
+    }
+    TORCH_CHECK(out.is_contiguous(), "out must be contiguous");
+    float *lse_ptr = nullptr;
+    if (is_training) {
+        TORCH_CHECK(lse.has_value() && lse->defined(), "is_training=True needs an lse tensor");
+        TORCH_CHECK(lse->device() == q.device() && lse->scalar_type() == at::kFloat &&
+                        lse->dim() == 3 && lse->size(0) == B && lse->size(1) == H &&
+                        lse->size(2) == N && lse->is_contiguous(),
+                    "lse must be a contiguous float32 [B, H, N] tensor on q's device");
+        lse_ptr = lse->data_ptr<float>();
+    }
+    const int64_t msb = mask.size(0) == 1 ? 0 : mask.size(1) * N * N;
+    const int64_t msh = mask.size(1) == 1 ? 0 : N * N;
+    const c10::DeviceGuard guard(q.device());
+    hipStream_t stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
+    const int st = sma_attn_fwd_bool_mask(q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                          reinterpret_cast<const uint8_t *>(mask.data_ptr<bool>()), msb, msh,
+                                          out.data_ptr(), lse_ptr, (int)B, (int)H, (int)N, (int)D, (float)scale,
+                                          dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
+    check_status(st, "sma_attn_fwd_bool_mask");
+}
+
 // backward(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, scale) -> None, the call the
 // reference's autograd function makes (python/sparse_attention.py:91-94) to a function its
 // binding never had.  dq, dk, dv are overwritten (not accumulated into).
@@ -175,6 +233,13 @@ PYBIND11_MODULE(sparse_attn_cuda, m)
     m.def("backward", &backward, "Sparse-mask attention backward (dq, dk, dv are overwritten)",
           py::arg("dout"), py::arg("q"), py::arg("k"), py::arg("v"), py::arg("out"), py::arg("lse"),
           py::arg("mask_packed"), py::arg("dq"), py::arg("dk"), py::arg("dv"), py::arg("scale"));
+    m.def("forward_bool_mask", &forward_bool_mask,
+          "Sparse-mask attention forward straight from the bool mask (one launch; see bool_mask_supported)",
+          py::arg("q"), py::arg("k"), py::arg("v"), py::arg("mask"), py::arg("out"), py::arg("lse"),
+          py::arg("scale"), py::arg("is_training"));
+    m.def("bool_mask_supported", &bool_mask_supported,
+          "Whether forward_bool_mask applies to these tensors (else use pack_mask + forward)", py::arg("q"),
+          py::arg("k"), py::arg("v"), py::arg("mask"));
     m.def("pack_mask", &pack_mask, "Pack a bool mask into uint32 words (returned as int32)",
           py::arg("mask"));
     m.def("version", []() { return sma_version(); });

@@ -165,6 +165,48 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
     a.H = H;
     a.N = N;
     a.D = D;
+    a.byte_mask = 0;
+    a.qtiles = (int)qtiles;
+    split_scale(scale, &a.q_scale, &a.post_mul);
+    last_tile_masks(N, &a.last_mask0, &a.last_mask1);
+
+    const hipError_t e = sma::launch_attn_fwd(a, dtype == SMA_DTYPE_BF16, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
+}
+
+int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const uint8_t *mask,
+                           int64_t mask_stride_b, int64_t mask_stride_h, void *out, float *lse,
+                           int B, int H, int N, int D, float scale, int dtype, void *stream)
+{
+    if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
+    if (D != 32 && D != 64) return SMA_ERR_HEAD_DIM;
+    if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
+    if (!isfinite(scale)) return SMA_ERR_SCALE;
+    const long long BH = (long long)B * H;
+    if (BH == 0 || N == 0) return SMA_OK;
+    if (!mask) return SMA_ERR_NULL_POINTER;
+    if (N % 64 != 0) return SMA_ERR_BAD_SHAPE;
+    const long long qtiles = (N + 127) / 128;
+    if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
+    // a lane's byte offset into the mask of one (b,h) is a 32-bit register
+    if ((long long)N * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
+    if (misaligned(mask, 16) || (lse && misaligned(lse, 4))) return SMA_ERR_ALIGNMENT;
+    if (mask_stride_b < 0 || mask_stride_h < 0 || ((mask_stride_b | mask_stride_h) & 15)) return SMA_ERR_STRIDE;
+
+    sma::AttnArgs a;
+    const sma_tensor t[4] = {dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D), dense(out, H, N, D)};
+    sma::Rows *to[4] = {&a.q, &a.k, &a.v, &a.out};
+    for (int i = 0; i < 4; ++i) {
+        const int st = to_rows(&t[i], N, D, to[i]);
+        if (st != SMA_OK) return st;
+    }
+    a.mask = sma::PackedMask{reinterpret_cast<const uint32_t *>(mask), mask_stride_b, mask_stride_h};
+    a.lse = lse;
+    a.BH = (int)BH;
+    a.H = H;
+    a.N = N;
+    a.D = D;
+    a.byte_mask = 1;
     a.qtiles = (int)qtiles;
     split_scale(scale, &a.q_scale, &a.post_mul);
     last_tile_masks(N, &a.last_mask0, &a.last_mask1);

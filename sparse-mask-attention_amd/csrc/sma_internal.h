@@ -46,11 +46,12 @@ __host__ __device__ inline uint32_t fastdiv(uint32_t n, FastDiv f)
 // Arguments of the fused forward kernel, already validated by the C-ABI layer.
 struct AttnArgs {
     Rows q, k, v;                   // inputs (never written)
-    PackedMask mask;
+    PackedMask mask;                // byte_mask != 0: p names boolean bytes [Bm, Hm, N, N], strides in bytes
     Rows out;
     float *lse;                     // [BH, N] contiguous, or nullptr
     int BH, H, N;
     int D;                          // head dim: 32, 64 or 128
+    int byte_mask;                  // the mask is the caller's boolean tensor, not packed words
     int qtiles;                     // ceil(N / 128): query tiles (work-groups) per (b,h)
     FastDiv div_qtiles, div_H;      // filled in by the launcher
     // exp(scale * s) is evaluated as exp2(post_mul * (q_scale * q) . k): q is multiplied by

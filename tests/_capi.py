@@ -55,6 +55,8 @@ def load():
         lib.sma_attn_fwd_strided.argtypes = [tp, tp, tp, vp, i64, i64, tp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_bwd_strided.restype = ci
         lib.sma_attn_bwd_strided.argtypes = [tp] * 5 + [vp, vp, i64, i64, tp, tp, tp, vp, ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_attn_fwd_bool_mask.restype = ci
+        lib.sma_attn_fwd_bool_mask.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         _lib = lib
     return _lib
 
@@ -150,3 +152,26 @@ def attn_bwd_strided(dout, q, k, v, out, lse, packed, grads=None, scale=None):
                                   ts[5], ts[6], ts[7], delta.data_ptr(), B, H, N, D, scale, dt, _stream())
     assert st == SMA_OK, lib.sma_strerror(st)
     return dq, dk, dv, delta
+
+
+def attn_fwd_bool_mask(q, k, v, mask, scale=None, want_lse=False, expect=SMA_OK):
+    """Forward straight from the boolean mask ([1|B, 1|H, N, N], contiguous) through
+    sma_attn_fwd_bool_mask; returns out (and lse), or the status if `expect` is an error code."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    assert mask.dtype == torch.bool and mask.is_contiguous()
+    Bm, Hm = mask.shape[:2]
+    msb = Hm * N * N if Bm == B and B > 1 else 0
+    msh = N * N if Hm == H and H > 1 else 0
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device) if want_lse else None
+    st = lib.sma_attn_fwd_bool_mask(q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), msb, msh,
+                                    out.data_ptr(), lse.data_ptr() if want_lse else None, B, H, N, D, scale, dt,
+                                    _stream())
+    if expect != SMA_OK:
+        return st
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return (out, lse) if want_lse else out

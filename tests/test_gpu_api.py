@@ -290,3 +290,31 @@ def test_expanded_mask_is_packed_once(sa, dev, monkeypatch):
     ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), small.cpu().expand(B, H, N, N))
     assert torch.allclose(out.float().cpu(), ref, atol=1e-2, rtol=1e-2)
     assert torch.equal(out, out_h)
+
+
+def test_inference_entry_point_reads_the_bool_mask_itself(sa, dev, monkeypatch):
+    """For shapes the single-launch kernel takes, sparse_attention_func must not pack the mask, and
+    must return exactly what the packing path returns; other shapes still go through pack_mask."""
+    calls = []
+    real = sa.pack_mask
+    monkeypatch.setattr(sa, "pack_mask", lambda m: (calls.append(tuple(m.shape)), real(m))[1])
+    q, k, v, mask = _inputs(2, 3, 192, torch.float16, 16)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    out = sa.sparse_attention_func(qd, kd, vd, md)
+    assert calls == []
+    assert torch.equal(out, sa.sparse_attention_func(qd, kd, vd, None, mask_packed=real(md)))
+    assert torch.equal(out, sa.sparse_attention(qd, kd, vd, md))
+    shared = sa.sparse_attention_func(qd, kd, vd, md[:1, :1].expand(2, 3, 192, 192))      # expanded view: read once
+    assert calls == [(2, 3, 192, 192)]                  # only the autograd call above packed
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask[:1, :1].expand(2, 3, 192, 192))
+    assert torch.allclose(shared.float().cpu(), ref, atol=1e-2, rtol=1e-2)
+    calls.clear()
+    q, k, v, mask = _inputs(1, 2, 100, torch.float16, 17)                                   # N % 64 != 0
+    sa.sparse_attention_func(q.to(dev), k.to(dev), v.to(dev), mask.to(dev))
+    assert calls == [(1, 2, 100, 100)]
+    # fp32 inputs: computed in bf16 through the same path, returned as fp32
+    q, k, v, mask = _inputs(1, 2, 128, torch.float32, 18)
+    o32 = sa.sparse_attention_func(q.to(dev), k.to(dev), v.to(dev), mask.to(dev))
+    assert o32.dtype == torch.float32
+    ref = O.sparse_attention_ref(q.bfloat16().float(), k.bfloat16().float(), v.bfloat16().float(), mask)
+    assert torch.allclose(o32.cpu(), ref, atol=1e-2, rtol=2e-2)

@@ -1,0 +1,107 @@
+"""GPU parity of sma_attn_fwd_bool_mask (the forward that reads the boolean mask itself) against
+sma_pack_mask + sma_attn_fwd: the arithmetic is the same kernel, only the source of the mask words
+differs, so the results must agree bit for bit; the pair is in turn checked against the oracle by
+the other test files (and once more here)."""
+import math
+
+import pytest
+import torch
+
+import _capi
+from oracle import sma_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(B, H, N, D, dtype, seed, keep=0.25):
+    g = torch.Generator().manual_seed(seed)
+    q, k, v = [torch.randn(B, H, N, D, generator=g).to(dtype) for _ in range(3)]
+    mask = torch.rand(B, H, N, N, generator=g) < keep
+    return q, k, v, mask
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [32, 64])
+@pytest.mark.parametrize("N", [64, 128, 192, 256, 512, 1024])
+def test_equals_pack_then_attention(dev, dtype, D, N):
+    B, H = 2, 3
+    q, k, v, mask = _inputs(B, H, N, D, dtype, 300 + N + D)
+    mask[0, 1, 5, :] = False                       # a row that keeps nothing
+    mask[1, 2, :, N - 1] = False                   # a key nobody keeps
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    want, want_lse = _capi.attn_fwd(qd, kd, vd, _capi.pack_mask(md), want_lse=True)
+    got, lse = _capi.attn_fwd_bool_mask(qd, kd, vd, md, want_lse=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and torch.equal(lse, want_lse)
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    assert torch.allclose(got.float().cpu(), ref, atol=1e-2, rtol=2e-2)
+    assert (got[0, 1, 5] == 0).all() and lse[0, 1, 5].item() == -math.inf
+
+
+@pytest.mark.parametrize("kind", ["all_true", "all_false", "diag", "block64", "causal", "columns"])
+def test_structured_masks(dev, kind):
+    B, H, N, D, dtype = 1, 2, 320, 64, torch.float16
+    q, k, v, _ = _inputs(B, H, N, D, dtype, 41)
+    if kind == "all_true":
+        mask = torch.ones(B, H, N, N, dtype=torch.bool)
+    elif kind == "all_false":
+        mask = torch.zeros(B, H, N, N, dtype=torch.bool)
+    elif kind == "diag":
+        mask = torch.eye(N, dtype=torch.bool).expand(B, H, N, N).contiguous()
+    elif kind == "block64":
+        g = torch.Generator().manual_seed(3)
+        blocks = torch.rand(B, H, N // 64, N // 64, generator=g) < 0.3
+        mask = blocks.repeat_interleave(64, dim=2).repeat_interleave(64, dim=3)
+    elif kind == "causal":
+        mask = torch.tril(torch.ones(N, N, dtype=torch.bool)).expand(B, H, N, N).contiguous()
+    else:                                           # every key position in turn, one per row: bit order
+        mask = torch.zeros(B, H, N, N, dtype=torch.bool)
+        idx = torch.arange(N)
+        mask[:, :, idx, (idx * 7 + 3) % N] = True
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    want = _capi.attn_fwd(qd, kd, vd, _capi.pack_mask(md))
+    got = _capi.attn_fwd_bool_mask(qd, kd, vd, md)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    if kind == "columns":                           # one kept key per row: out is that row of v, exactly
+        idx = torch.arange(N)
+        assert torch.equal(got.cpu(), v[:, :, (idx * 7 + 3) % N])
+
+
+@pytest.mark.parametrize("shape", ["11", "B1", "1H"])
+def test_shared_masks(dev, shape):
+    B, H, N, D = 3, 4, 128, 64
+    Bm, Hm = (1 if shape[0] == "1" else B), (1 if shape[1] == "1" else H)
+    q, k, v, _ = _inputs(B, H, N, D, torch.bfloat16, 52)
+    g = torch.Generator().manual_seed(6)
+    small = torch.rand(Bm, Hm, N, N, generator=g) < 0.3
+    qd, kd, vd = (t.to(dev) for t in (q, k, v))
+    want = _capi.attn_fwd(qd, kd, vd, _capi.pack_mask(small.expand(B, H, N, N).contiguous().to(dev)))
+    got = _capi.attn_fwd_bool_mask(qd, kd, vd, small.to(dev))
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+
+
+def test_scales_many_heads_and_long_rows(dev):
+    q, k, v, mask = _inputs(1, 2, 256, 64, torch.float16, 61)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    packed = _capi.pack_mask(md)
+    for scale in (1.0, -0.3, 0.01):                 # scale 1 takes the post-multiplied exponent
+        assert torch.equal(_capi.attn_fwd_bool_mask(qd, kd, vd, md, scale=scale),
+                           _capi.attn_fwd(qd, kd, vd, packed, scale=scale))
+    q, k, v, mask = _inputs(8, 40, 256, 64, torch.float16, 62)      # several rounds of work-groups
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    assert torch.equal(_capi.attn_fwd_bool_mask(qd, kd, vd, md), _capi.attn_fwd(qd, kd, vd, _capi.pack_mask(md)))
+    q, k, v, mask = _inputs(1, 2, 2112, 64, torch.float16, 63, keep=0.1)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    assert torch.equal(_capi.attn_fwd_bool_mask(qd, kd, vd, md), _capi.attn_fwd(qd, kd, vd, _capi.pack_mask(md)))
+    torch.cuda.synchronize()
+
+
+def test_limits_are_reported(dev):
+    q, k, v, mask = _inputs(1, 1, 100, 64, torch.float16, 70)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    assert _capi.attn_fwd_bool_mask(qd, kd, vd, md, expect=_capi.SMA_ERR_BAD_SHAPE) == _capi.SMA_ERR_BAD_SHAPE
+    q, k, v, mask = _inputs(1, 1, 64, 128, torch.float16, 71)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    assert _capi.attn_fwd_bool_mask(qd, kd, vd, md, expect=_capi.SMA_ERR_HEAD_DIM) == _capi.SMA_ERR_HEAD_DIM

@@ -22,7 +22,7 @@ def test_library_exports_every_declared_symbol(capi):
     header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
     declared = set(re.findall(r"\b(sma_[a-z_0-9]+)\s*\(", header))
     assert {"sma_version", "sma_strerror", "sma_pack_mask", "sma_attn_fwd", "sma_attn_bwd",
-            "sma_attn_fwd_strided", "sma_attn_bwd_strided"} <= declared
+            "sma_attn_fwd_strided", "sma_attn_bwd_strided", "sma_attn_fwd_bool_mask"} <= declared
     for name in declared:
         assert hasattr(capi, name), f"{name} is declared in sma.h but not exported"
     assert capi.sma_version() >= 100
@@ -73,6 +73,21 @@ def test_argument_validation_needs_no_gpu(capi):
     assert scall(msh=-1) == _capi.SMA_ERR_STRIDE
     assert scall(q=None) == _capi.SMA_ERR_NULL_POINTER
     assert scall(B=0) == _capi.SMA_OK
+
+    # forward straight from the boolean mask: limits are reported, not worked around
+    fb = capi.sma_attn_fwd_bool_mask
+
+    def bcall(mask=p, msb=4096, msh=4096, **kw):
+        a = dict(ok_args, **kw)
+        return fb(p, p, p, mask, msb, msh, p, None, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
+
+    assert bcall(D=128) == _capi.SMA_ERR_HEAD_DIM
+    assert bcall(N=100) == _capi.SMA_ERR_BAD_SHAPE                            # not a multiple of 64
+    assert bcall(mask=None) == _capi.SMA_ERR_NULL_POINTER
+    assert bcall(mask=ctypes.c_void_p(0x1004)) == _capi.SMA_ERR_ALIGNMENT
+    assert bcall(msh=24) == _capi.SMA_ERR_STRIDE
+    assert bcall(dtype=5) == _capi.SMA_ERR_DTYPE
+    assert bcall(B=0) == _capi.SMA_OK
 
     g = capi.sma_pack_mask
     assert g(None, p, 1, 1, 8, None) == _capi.SMA_ERR_NULL_POINTER
