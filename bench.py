@@ -2,13 +2,20 @@
 """Benchmark of the sparse-mask attention hot path on one MI355X.
 
 A step is one pass of the hot path over one batch of synthetic input, as the reference times it
-(run.py:147-155, :172-183): pack_mask(bool mask) -> allocate out -> fused attention forward, called
-through the `sparse_attn_cuda` module with all inputs already resident in HBM.  The headline
-value is dense-equivalent TFLOP/s, 4*B*H*N*N*D per step whatever the sparsity (run.py:198-203).
+(run.py:147-155, :172-183): boolean mask in, attention output out, called through the
+`sparse_attn_cuda` module with all inputs already resident in HBM.  The reference needs two
+launches for it (pack_mask, then the fused forward); here the step is: allocate out -> ONE launch
+that reads the boolean mask itself (forward_bool_mask), where the kernel's limits allow (head dim
+32 or 64, N a multiple of 64), else pack_mask -> allocate out -> forward.  The two-launch step is
+timed as well and reported beside it.  The headline value is dense-equivalent TFLOP/s,
+4*B*H*N*N*D per step whatever the sparsity (run.py:198-203).
 
 Prints ONE JSON line.  Besides the whole-step figure it carries
-  roofline      the fused attention kernel alone (the dominant kernel) against the dense FP16 MFMA
-                peak, from stream-event timing of back-to-back launches on the launch stream;
+  roofline      the dominant kernel of the step alone, from stream-event timing of back-to-back
+                launches on the launch stream: the forward that reads the boolean mask (100.7 MB of
+                compulsory traffic for 12.9 GFLOP on the headline workload, 128 FLOP/B, i.e. on the
+                HBM side of the roofline) or, where that does not apply, the packed-mask forward;
+  roofline_attn the packed-mask forward kernel alone against the dense FP16 MFMA peak;
   roofline_pack the packer alone against the HBM peak;
   roofline_bwd  the backward (its two kernels, one call) against the MFMA peak, 2.5 x the forward's FLOP;
   cpu_baseline  the oracle's PyTorch formulation of the same workload on the host cores.
@@ -103,21 +110,33 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    def step():
+    def step_two_launches():
         packed = ext.pack_mask(md)
         out = torch.empty_like(qd)
         ext.forward(qd, kd, vd, packed, out, None, scale, False)
         return out
 
-    # ---- whole step: W untimed, K timed, synchronize on both sides ----
-    for _ in range(args.warmup):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
+    def step_one_launch():
+        out = torch.empty_like(qd)
+        ext.forward_bool_mask(qd, kd, vd, md, out, None, scale, False)
+        return out
+
+    one_launch = bool(ext.bool_mask_supported(qd, kd, vd, md))
+    step = step_one_launch if one_launch else step_two_launches
+
+    def wall_ms(fn):
+        """W untimed, K timed calls, synchronize on both sides."""
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    two_launch_ms = wall_ms(step_two_launches)
+    ms_per_step = wall_ms(step) if one_launch else two_launch_ms
     value = w.dense_flops / (ms_per_step * 1e-3) / 1e12
 
     # ---- the two kernels on their own: back-to-back launches between stream events ----
@@ -133,6 +152,9 @@ def main():
     pack_ms = event_time_ms(lambda: lib.sma_pack_mask(md.data_ptr(), packed.data_ptr(), w.B, w.H, w.N, stream),
                             10, reps, torch)
     api_ms = event_time_ms(lambda: sa.sparse_attention_func(qd, kd, vd, md), 10, reps, torch)
+    fused_ms = None
+    if one_launch:
+        fused_ms = event_time_ms(lambda: ext.forward_bool_mask(qd, kd, vd, md, out, None, scale, False), 10, reps, torch)
     # the backward (dQ kernel, then dK/dV kernel) on the forward's saved out and lse
     lse = torch.empty(w.B, w.H, w.N, dtype=torch.float32, device=dev)
     ext.forward(qd, kd, vd, packed, out, lse, scale, True)
@@ -166,8 +188,12 @@ def main():
         "dtype": "fp16" if w.dtype == torch.float16 else "bf16",
         "data": "synthetic",
         "config": {"workload": f"{w.name}: B={w.B} H={w.H} N={w.N} D={w.D} {w.mask_kind} mask keep_p={w.keep_prob}",
-                   "step": "pack_mask + torch.empty_like + fused forward via sparse_attn_cuda (no LSE)",
+                   "step": ("torch.empty_like + forward_bool_mask via sparse_attn_cuda (bool mask in, one launch, no LSE)"
+                            if one_launch else
+                            "pack_mask + torch.empty_like + forward via sparse_attn_cuda (no LSE)"),
                    "dense_equiv_flop_per_step": w.dense_flops},
+        "step_pack_then_attention_ms": round(two_launch_ms, 5),
+        "step_pack_then_attention_tflops": round(w.dense_flops / (two_launch_ms * 1e-3) / 1e12, 3),
         "attn_kernel_ms": round(attn_ms, 5),
         "attn_kernel_tflops": round(attn_tflops, 2),
         "attn_kernel_hbm_gbps": round(w.attn_bytes / (attn_ms * 1e-3) / 1e9, 1),
@@ -176,10 +202,10 @@ def main():
         "pack_kernel_ms": round(pack_ms, 5),
         "backward_ms": round(bwd_ms, 5),
         "api_sparse_attention_func_ms": round(api_ms, 5),
-        "roofline": {"kernel": "attn_fwd_kernel", "bound": "mfma", "achieved": round(attn_tflops, 2),
-                     "peak": harness.MI355X_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(attn_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4),
-                     "traffic": measured_traffic(w.name, "attn_fwd_kernel"), "algorithmic_bytes": w.attn_bytes},
+        "roofline_attn": {"kernel": "attn_fwd_kernel (packed mask)", "bound": "mfma", "achieved": round(attn_tflops, 2),
+                          "peak": harness.MI355X_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
+                          "frac": round(attn_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4),
+                          "traffic": measured_traffic(w.name, "attn_fwd_kernel"), "algorithmic_bytes": w.attn_bytes},
         "roofline_pack": {"kernel": "pack_flat_kernel" if w.N % 32 == 0 else ("pack_row8_kernel" if w.N % 8 == 0 else "pack_rows_kernel"),
                           "bound": "hbm", "achieved": round(pack_gbps, 1), "peak": harness.MI355X_HBM_GBPS,
                           "unit": "GB/s", "frac": round(pack_gbps / harness.MI355X_HBM_GBPS, 4),
@@ -189,6 +215,21 @@ def main():
                          "unit": "TFLOP/s", "frac": round(bwd_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4),
                          "traffic": measured_traffic(w.name, "attn_bwd_dq_kernel", "attn_bwd_dkv_kernel"), "algorithmic_bytes": w.bwd_bytes},
     }
+
+    if one_launch:
+        gbps = w.fused_bytes / (fused_ms * 1e-3) / 1e9
+        tfl = w.dense_flops / (fused_ms * 1e-3) / 1e12
+        result["fused_kernel_ms"] = round(fused_ms, 5)
+        result["roofline"] = {"kernel": "attn_fwd_kernel (boolean mask in)", "bound": "hbm", "achieved": round(gbps, 1),
+                              "peak": harness.MI355X_HBM_GBPS, "unit": "GB/s",
+                              "frac": round(gbps / harness.MI355X_HBM_GBPS, 4),
+                              "traffic": measured_traffic(w.name, "attn_fwd_bool_mask_kernel"),
+                              "algorithmic_bytes": w.fused_bytes,
+                              "flop_per_byte": round(w.dense_flops / w.fused_bytes, 1),
+                              "mfma_tflops": round(tfl, 2),
+                              "mfma_frac": round(tfl / harness.MI355X_MFMA_F16_TFLOPS, 4)}
+    else:
+        result["roofline"] = dict(result["roofline_attn"])
 
     if not args.no_cpu_baseline:
         from oracle import sma_oracle

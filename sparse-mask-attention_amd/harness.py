@@ -50,6 +50,12 @@ class Workload:
         return 4 * self.B * self.H * self.N * self.D * 2 + 4 * self.B * self.H * self.N * self.n_words
 
     @property
+    def fused_bytes(self) -> int:
+        """Algorithmic bytes of the forward that reads the boolean mask itself: q, k, v, out and one
+        byte per score."""
+        return 4 * self.B * self.H * self.N * self.D * 2 + self.B * self.H * self.N * self.N
+
+    @property
     def bwd_dense_flops(self) -> int:
         """Dense-equivalent FLOP of the backward, by the usual convention 2.5 x the forward: the five
         N x N x D products dV, dP, dQ, dK and the recomputed S (what the kernels execute is seven,
