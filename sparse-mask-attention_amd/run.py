@@ -8,8 +8,10 @@ its competitor baselines (Triton, cuDNN, FlashInfer, flash-attn):
                sparsity, N in {64,128,256,512}, max |out - fp32 PyTorch formulation| < 1e-2, and the
                fully-masked-row case (N=8, row 0 masked) which must contain no NaN;
 * perf         the N-sweep at B=16 and the B-sweep at N=512 (run.py:410-450), H=12, D=64, fp16,
-               75 % sparsity; every latency covers pack_mask + output allocation + the fused kernel,
-               10 warm-up and 50 timed calls between stream events (run.py:172-183), with
+               75 % sparsity; every latency covers what the reference's covers, boolean mask in and
+               output out (there: pack_mask + allocation + forward; here: allocation + the one
+               launch that reads the boolean mask, with the reference's three calls in a second
+               column), 10 warm-up and 50 timed calls between stream events (run.py:172-183), with
                dense-equivalent TFLOP/s and percent of the MI355X dense FP16 MFMA peak.
 
 Inputs are generated on the CPU from an explicit seed and moved to the GPU.  The PyTorch
@@ -33,12 +35,23 @@ import harness  # noqa: E402
 sa = importlib.import_module("python.sparse_attention")
 
 
-def sparse_attention_hip_fwd(q, k, v, mask):
-    """pack_mask + allocation + fused forward: what the reference times (run.py:147-155)."""
+def sparse_attention_hip_two_launches(q, k, v, mask):
+    """pack_mask + allocation + forward: the reference's sequence of calls (run.py:147-155)."""
     import sparse_attn_cuda as ext
     packed = ext.pack_mask(mask)
     out = torch.empty_like(q)
     ext.forward(q, k, v, packed, out, None, 1.0 / math.sqrt(q.shape[-1]), False)
+    return out
+
+
+def sparse_attention_hip_fwd(q, k, v, mask):
+    """Boolean mask in, output out: allocation + the forward that reads the boolean mask itself
+    where it applies (head dim 32 / 64, N a multiple of 64), else the two launches above."""
+    import sparse_attn_cuda as ext
+    if not ext.bool_mask_supported(q, k, v, mask):
+        return sparse_attention_hip_two_launches(q, k, v, mask)
+    out = torch.empty_like(q)
+    ext.forward_bool_mask(q, k, v, mask, out, None, 1.0 / math.sqrt(q.shape[-1]), False)
     return out
 
 
@@ -81,20 +94,22 @@ def run_perf(device):
     peak = harness.MI355X_MFMA_F16_TFLOPS
     print("=" * 56 + f"\nperformance (fp16, H=12, D=64, sparsity 0.75; peak {peak} TFLOP/s)\n" + "=" * 56)
     print("\n[sequence length sweep]  B=16")
-    print(f"  {'N':>6}  {'latency(ms)':>12}  {'TFLOPS':>8}  {'MFU%':>7}  {'torch SDPA(ms)':>15}  {'speed-up':>8}")
+    print(f"  {'N':>6}  {'latency(ms)':>12}  {'TFLOPS':>8}  {'MFU%':>7}  {'pack+fwd(ms)':>13}  {'torch SDPA(ms)':>15}  {'speed-up':>8}")
     for N in (64, 128, 256, 512, 1024):
         q, k, v, mask = _inputs(16, 12, N, 1, device)
         lat = harness.measure_latency(lambda: sparse_attention_hip_fwd(q, k, v, mask))
+        two = harness.measure_latency(lambda: sparse_attention_hip_two_launches(q, k, v, mask))
         tf, mfu = harness.compute_mfu(lat, 16, 12, N, 64, peak)
         ref = harness.measure_latency(lambda: sdpa_bool_mask(q, k, v, mask))
-        print(f"  {N:>6}  {lat:>12.4f}  {tf:>8.2f}  {mfu:>7.1f}%  {ref:>15.4f}  {ref / lat:>7.1f}x")
+        print(f"  {N:>6}  {lat:>12.4f}  {tf:>8.2f}  {mfu:>7.1f}%  {two:>13.4f}  {ref:>15.4f}  {ref / lat:>7.1f}x")
     print("\n[batch size sweep]  N=512")
-    print(f"  {'B':>6}  {'latency(ms)':>12}  {'TFLOPS':>8}  {'MFU%':>7}  {'seq/s':>10}")
+    print(f"  {'B':>6}  {'latency(ms)':>12}  {'TFLOPS':>8}  {'MFU%':>7}  {'pack+fwd(ms)':>13}  {'seq/s':>10}")
     for B in (1, 4, 8, 16, 32, 64):
         q, k, v, mask = _inputs(B, 12, 512, 2, device)
         lat = harness.measure_latency(lambda: sparse_attention_hip_fwd(q, k, v, mask))
+        two = harness.measure_latency(lambda: sparse_attention_hip_two_launches(q, k, v, mask))
         tf, mfu = harness.compute_mfu(lat, B, 12, 512, 64, peak)
-        print(f"  {B:>6}  {lat:>12.4f}  {tf:>8.2f}  {mfu:>7.1f}%  {B / (lat / 1e3):>10.0f}")
+        print(f"  {B:>6}  {lat:>12.4f}  {tf:>8.2f}  {mfu:>7.1f}%  {two:>13.4f}  {B / (lat / 1e3):>10.0f}")
     print()
 
 
