@@ -127,18 +127,21 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     const uint32_t q_rb = 2u * q_sn, k_rb = 2u * k_sn, v_rb = 2u * v_sn;                   // row pitch, bytes
 
     // ---- mask words: wave-private async copies, slot = tile % NSTAGE, lane i -> (row i/2, word i%2) ----
-    // BYTEMASK (N % 64 == 0): the wave's 32 x 64 bytes of a tile as two copies of 16 rows; lane i
+    // BYTEMASK (N % 16 == 0): the wave's 32 x 64 bytes of a tile as two copies of 16 rows; lane i
     // fills (row 16j + i/4, position i%4) with the global 16-byte chunk position ^ ((row >> 2) & 3),
-    // which makes the reads below (lane = row, two chunks each) free of bank conflicts.
+    // which makes the reads below (lane = row, two chunks each) free of bank conflicts.  In a last
+    // tile of fewer than 64 keys the chunks beyond the row's end re-read its first chunk; their
+    // bits are cleared with the pad bits below.
     const int mrow = BYTEMASK ? 0 : qt * BM + wave * 32 + (lane >> 1);
     const uint32_t m_voff = BYTEMASK ? 0u : (uint32_t)(((size_t)(mrow < N ? mrow : N - 1) * nw + (lane & 1)) * 4);
-    uint32_t mb_voff[2] = {0u, 0u};
+    uint32_t mb_voff[2] = {0u, 0u}, mb_chunk[2] = {0u, 0u};
     if constexpr (BYTEMASK) {
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int row = 16 * j + (lane >> 2);
             const int grow = qt * BM + wave * 32 + row;
-            mb_voff[j] = (uint32_t)(grow < N ? grow : N - 1) * (uint32_t)N + (uint32_t)(((lane & 3) ^ ((row >> 2) & 3)) << 4);
+            mb_chunk[j] = (uint32_t)(((lane & 3) ^ ((row >> 2) & 3)) << 4);
+            mb_voff[j] = (uint32_t)(grow < N ? grow : N - 1) * (uint32_t)N + mb_chunk[j];
         }
     }
     const uint32_t mask_dst = lds0 + wave * (BYTEMASK ? 2048 : 256);
@@ -146,8 +149,15 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         constexpr int SLOT = decltype(slot_c)::value;
         if constexpr (BYTEMASK) {
             const uint8_t *src = reinterpret_cast<const uint8_t *>(mb) + (size_t)x * BN;
-            async_copy_b128_at<OFF_MASK + SLOT * MASK_SLOT>(mask_dst, src, mb_voff[0]);
-            async_copy_b128_at<OFF_MASK + SLOT * MASK_SLOT + 1024>(mask_dst, src, mb_voff[1]);
+            uint32_t vo[2] = {mb_voff[0], mb_voff[1]};
+            if (ragged && x == T - 1) {
+                const uint32_t row_end = (uint32_t)(N - x * BN);       // bytes of the row left in this tile
+#pragma unroll
+                for (int j = 0; j < 2; ++j)
+                    if (mb_chunk[j] >= row_end) vo[j] -= mb_chunk[j];
+            }
+            async_copy_b128_at<OFF_MASK + SLOT * MASK_SLOT>(mask_dst, src, vo[0]);
+            async_copy_b128_at<OFF_MASK + SLOT * MASK_SLOT + 1024>(mask_dst, src, vo[1]);
         } else {
             uint32_t voff = m_voff;
             if (2 * x + 1 >= nw) voff -= (lane & 1) * 4;           // odd word count: re-read the last word
@@ -557,7 +567,7 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     }
     if (a.byte_mask) {
         // built for contiguous rows and head dims 32 and 64 only (checked by the C-ABI layer)
-        if (!packed || D == 2 * HD || (a.N & (BN - 1)) != 0) return hipErrorInvalidValue;
+        if (!packed || D == 2 * HD || (a.N & 15) != 0) return hipErrorInvalidValue;
         if (D == 32) { SMA_FWD_BYTEMASK_VARIANTS(32) } else { SMA_FWD_BYTEMASK_VARIANTS(64) }
     } else if (D == 32) { SMA_FWD_VARIANTS(32) } else if (D == 64) { SMA_FWD_VARIANTS(64) } else { SMA_FWD_VARIANTS(128) }
 #undef SMA_FWD_VARIANTS

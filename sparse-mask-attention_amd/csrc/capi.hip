@@ -185,7 +185,7 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
     const long long BH = (long long)B * H;
     if (BH == 0 || N == 0) return SMA_OK;
     if (!mask) return SMA_ERR_NULL_POINTER;
-    if (N % 64 != 0) return SMA_ERR_BAD_SHAPE;
+    if (N % 16 != 0) return SMA_ERR_BAD_SHAPE;          // rows of the mask must start 16-byte aligned
     const long long qtiles = (N + 127) / 128;
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
     // a lane's byte offset into the mask of one (b,h) is a 32-bit register
