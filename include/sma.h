@@ -128,7 +128,7 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
  * boolean bytes themselves and forms the packed words of each 64-key tile on the fly, so the packing
  * pass, its launch and the round trip of the words through memory disappear.
  *
- *   q, k, v, out    contiguous [B,H,N,D], D = 32 or 64; N must be a multiple of 16
+ *   q, k, v, out    contiguous [B,H,N,D], D = 32, 64 or 128; N must be a multiple of 16
  *   mask            uint8 [Bm,Hm,N,N] with Bm in {1,B}, Hm in {1,H}, rows contiguous, 16-byte aligned;
  *                   every byte must be 0 or 1 (torch.bool storage; unlike sma_pack_mask, other
  *                   non-zero values are not accepted); mask_stride_b / mask_stride_h in BYTES,

@@ -75,9 +75,15 @@ template <int NH, bool BYTEMASK> struct Cfg {
     // LDS map (bytes)
     static constexpr int STAGE_BYTES = 2 * NH * TILE_BYTES;         // K halves, then V halves
     static constexpr int OFF_V = NH * TILE_BYTES;                   // V inside a stage
-    static constexpr int OFF_MASK = NSTAGE * STAGE_BYTES;           // NSTAGE slots x 4 waves x (64 words | 2 KiB of bytes)
-    static constexpr int MASK_SLOT = BYTEMASK ? 8192 : 1024;
-    static constexpr int OFF_LUT = OFF_MASK + NSTAGE * MASK_SLOT;   // 16 x 16 B
+    // mask: packed words in NSTAGE slots of 4 waves x 64 words; bytes in slots of 4 waves x 2 KiB,
+    // two of them for head dims up to 64 and, for want of LDS, ONE for 128: a wave has turned its
+    // bytes into words before it requests the next tile's (see the main loop), so one slot is
+    // enough, at the price of waiting for those reads before the requests (3 % on the headline
+    // workload, which is why two are used where they fit)
+    static constexpr int OFF_MASK = NSTAGE * STAGE_BYTES;
+    static constexpr int BYTE_SLOTS = NH == 1 ? 2 : 1;
+    static constexpr int MASK_SLOT = BYTEMASK ? (BYTE_SLOTS - 1) * 8192 : 1024;     // distance between the slots
+    static constexpr int OFF_LUT = OFF_MASK + (BYTEMASK ? BYTE_SLOTS * 8192 : NSTAGE * 1024);   // 16 x 16 B
     static constexpr int LDS_BYTES = OFF_LUT + 256;
 };
 
@@ -149,6 +155,8 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         constexpr int SLOT = decltype(slot_c)::value;
         if constexpr (BYTEMASK) {
             const uint8_t *src = reinterpret_cast<const uint8_t *>(mb) + (size_t)x * BN;
+            // a single slot is refilled: this wave's reads of the previous tile's bytes must be over
+            if constexpr (C::BYTE_SLOTS == 1) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             uint32_t vo[2] = {mb_voff[0], mb_voff[1]};
             if (ragged && x == T - 1) {
                 const uint32_t row_end = (uint32_t)(N - x * BN);       // bytes of the row left in this tile
@@ -566,9 +574,9 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     default: kernel = attn_fwd_kernel<true, true, true, HDIM, true>; break;            \
     }
     if (a.byte_mask) {
-        // built for contiguous rows and head dims 32 and 64 only (checked by the C-ABI layer)
-        if (!packed || D == 2 * HD || (a.N & 15) != 0) return hipErrorInvalidValue;
-        if (D == 32) { SMA_FWD_BYTEMASK_VARIANTS(32) } else { SMA_FWD_BYTEMASK_VARIANTS(64) }
+        // built for contiguous rows only (checked by the C-ABI layer)
+        if (!packed || (a.N & 15) != 0) return hipErrorInvalidValue;
+        if (D == 32) { SMA_FWD_BYTEMASK_VARIANTS(32) } else if (D == 64) { SMA_FWD_BYTEMASK_VARIANTS(64) } else { SMA_FWD_BYTEMASK_VARIANTS(128) }
     } else if (D == 32) { SMA_FWD_VARIANTS(32) } else if (D == 64) { SMA_FWD_VARIANTS(64) } else { SMA_FWD_VARIANTS(128) }
 #undef SMA_FWD_VARIANTS
 #undef SMA_FWD_BYTEMASK_VARIANTS

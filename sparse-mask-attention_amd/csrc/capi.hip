@@ -179,7 +179,7 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
                            int B, int H, int N, int D, float scale, int dtype, void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
-    if (D != 32 && D != 64) return SMA_ERR_HEAD_DIM;
+    if (D != 32 && D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
     if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
     if (!isfinite(scale)) return SMA_ERR_SCALE;
     const long long BH = (long long)B * H;

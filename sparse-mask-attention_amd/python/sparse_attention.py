@@ -33,7 +33,7 @@ What differs from the reference, on purpose:
   is computed exactly by zero-padding q, k, v to the next of these (the scores and the first D output
   columns do not change; the scale stays 1/sqrt(D)) at the price of the padding copies.
 * ``sparse_attention_func`` (no autograd, the mask is used once) does not pack the mask: where the
-  kernel's limits allow (contiguous q, k, v, head dim 32 or 64, N a multiple of 16) one launch reads
+  kernel's limits allow (contiguous q, k, v, N a multiple of 16) one launch reads
   the bool mask itself and forms the packed words tile by tile, which is 15-35 % faster than
   pack + attention; otherwise it packs as the reference does.  Results are bit-identical.
 * ``.backward()`` works.  The reference calls a ``sparse_attn_cuda.backward`` that was never

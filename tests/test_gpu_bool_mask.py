@@ -21,7 +21,7 @@ def _inputs(B, H, N, D, dtype, seed, keep=0.25):
 
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
-@pytest.mark.parametrize("D", [32, 64])
+@pytest.mark.parametrize("D", [32, 64, 128])
 @pytest.mark.parametrize("N", [16, 48, 64, 80, 128, 144, 192, 256, 400, 512, 1008, 1024])
 def test_equals_pack_then_attention(dev, dtype, D, N):
     B, H = 2, 3
@@ -102,6 +102,6 @@ def test_limits_are_reported(dev):
     q, k, v, mask = _inputs(1, 1, 104, 64, torch.float16, 70)                  # rows not 16-byte aligned
     qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
     assert _capi.attn_fwd_bool_mask(qd, kd, vd, md, expect=_capi.SMA_ERR_BAD_SHAPE) == _capi.SMA_ERR_BAD_SHAPE
-    q, k, v, mask = _inputs(1, 1, 64, 128, torch.float16, 71)
+    q, k, v, mask = _inputs(1, 1, 64, 96, torch.float16, 71)
     qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
     assert _capi.attn_fwd_bool_mask(qd, kd, vd, md, expect=_capi.SMA_ERR_HEAD_DIM) == _capi.SMA_ERR_HEAD_DIM

@@ -81,7 +81,7 @@ def test_argument_validation_needs_no_gpu(capi):
         a = dict(ok_args, **kw)
         return fb(p, p, p, mask, msb, msh, p, None, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
 
-    assert bcall(D=128) == _capi.SMA_ERR_HEAD_DIM
+    assert bcall(D=96) == _capi.SMA_ERR_HEAD_DIM
     assert bcall(N=100) == _capi.SMA_ERR_BAD_SHAPE                            # not a multiple of 16
     assert bcall(mask=None) == _capi.SMA_ERR_NULL_POINTER
     assert bcall(mask=ctypes.c_void_p(0x1004)) == _capi.SMA_ERR_ALIGNMENT
