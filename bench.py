@@ -5,8 +5,8 @@ A step is one pass of the hot path over one batch of synthetic input, as the ref
 (run.py:147-155, :172-183): boolean mask in, attention output out, called through the
 `sparse_attn_cuda` module with all inputs already resident in HBM.  The reference needs two
 launches for it (pack_mask, then the fused forward); here the step is: allocate out -> ONE launch
-that reads the boolean mask itself (forward_bool_mask), where the kernel's limits allow (head dim
-32 or 64, N a multiple of 16), else pack_mask -> allocate out -> forward.  The two-launch step is
+that reads the boolean mask itself (forward_bool_mask), where the kernel's limits allow (N a
+multiple of 16), else pack_mask -> allocate out -> forward.  The two-launch step is
 timed as well and reported beside it.  The headline value is dense-equivalent TFLOP/s,
 4*B*H*N*N*D per step whatever the sparsity (run.py:198-203).
 
