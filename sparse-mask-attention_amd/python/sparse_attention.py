@@ -201,6 +201,9 @@ def sparse_attention(q, k, v, mask, mask_packed=None):
     """
     _check_inputs(q, k, v, mask, mask_packed)
     _require_ext(q)
+    if not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)):
+        # nothing will be differentiated: no LSE, and the mask can be read without packing it
+        return sparse_attention_func(q, k, v, mask, mask_packed)
     B, H, N, D = q.shape
     scale = 1.0 / math.sqrt(D)
 

@@ -303,7 +303,12 @@ def test_inference_entry_point_reads_the_bool_mask_itself(sa, dev, monkeypatch):
     out = sa.sparse_attention_func(qd, kd, vd, md)
     assert calls == []
     assert torch.equal(out, sa.sparse_attention_func(qd, kd, vd, None, mask_packed=real(md)))
-    assert torch.equal(out, sa.sparse_attention(qd, kd, vd, md))
+    assert torch.equal(out, sa.sparse_attention(qd, kd, vd, md))            # nothing requires grad: same path
+    assert calls == []
+    leaves = [t.clone().requires_grad_(True) for t in (qd, kd, vd)]
+    assert torch.equal(out, sa.sparse_attention(*leaves, md))               # autograd: packs, saves the lse
+    with torch.no_grad():
+        assert torch.equal(out, sa.sparse_attention(*leaves, md))
     shared = sa.sparse_attention_func(qd, kd, vd, md[:1, :1].expand(2, 3, 192, 192))      # expanded view: read once
     assert calls == [(2, 3, 192, 192)]                  # only the autograd call above packed
     ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask[:1, :1].expand(2, 3, 192, 192))
