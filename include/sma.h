@@ -134,6 +134,9 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
  *                   non-zero values are not accepted); mask_stride_b / mask_stride_h in BYTES,
  *                   multiples of 16, 0 = shared between batch entries / heads
  *   lse             NULL or float [B,H,N]
+ *   packed_out      NULL, or uint32 [Bm,Hm,N,ceil(N/32)] (contiguous): receives exactly what
+ *                   sma_pack_mask would write for this mask, as a by-product, for callers who
+ *                   need the packed words afterwards (sma_attn_bwd)
  *
  * Anything outside these limits returns an error code and is served by sma_pack_mask followed by
  * sma_attn_fwd (or its strided form), which give the same results.
@@ -143,7 +146,8 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
  */
 int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const uint8_t *mask,
                            int64_t mask_stride_b, int64_t mask_stride_h, void *out, float *lse,
-                           int B, int H, int N, int D, float scale, int dtype, void *stream);
+                           uint32_t *packed_out, int B, int H, int N, int D, float scale, int dtype,
+                           void *stream);
 
 /* sma_attn_bwd for strided dout, q, k, v, out, dq, dk, dv and a shared mask (see
  * sma_attn_fwd_strided); lse and delta_ws are contiguous float [B,H,N].

@@ -172,6 +172,18 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
             async_copy_b32_at<OFF_MASK + SLOT * MASK_SLOT>(mask_dst, mb + 2 * x, voff);
         }
     };
+    // BYTEMASK: where this lane's row of packed words goes, if the caller wants them ([Bm, Hm, N, nw]
+    // like the mask; a mask shared between batch entries / heads is written by the first of them)
+    const int qrow = qt * BM + wave * 32 + l32;
+    uint32_t *words_out = nullptr;
+    if constexpr (BYTEMASK) {
+        const bool writer = (a.mask.sb != 0 || bi == 0) && (a.mask.sh != 0 || hi == 0);
+        if (a.mask_out != nullptr && writer) {
+            const int Hm = a.mask.sh != 0 ? a.H : 1;
+            const size_t slab_m = (size_t)((a.mask.sb != 0 ? bi : 0) * Hm + (a.mask.sh != 0 ? hi : 0));
+            words_out = a.mask_out + (slab_m * N + (qrow < N ? qrow : 0)) * nw;
+        }
+    }
     const uint32_t maddr = BYTEMASK ? lds0 + OFF_MASK + wave * 2048 + l32 * 64 : lds0 + OFF_MASK + wave * 256 + l32 * 8;
     const int msw = (l32 >> 2) & 3;
     auto mask_words = [&](int x, int slot) __attribute__((always_inline)) -> u32x2 {
@@ -188,17 +200,20 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
             b1 = __builtin_amdgcn_udot4(d0.w, 0x80402010u, b1, false);
             b2 = __builtin_amdgcn_udot4(d1.y, 0x80402010u, b2, false);
             b3 = __builtin_amdgcn_udot4(d1.w, 0x80402010u, b3, false);
-            const uint32_t mine = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            uint32_t mine = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            if (x == T - 1) mine &= hh ? a.last_mask1 : a.last_mask0;       // bits of keys >= N
+            // a caller who will need the packed words (for the backward) gets them as a by-product
+            if (words_out != nullptr && qrow < N && 2 * x + hh < nw) words_out[2 * x + hh] = mine;
             // lanes < 32 hold the word of keys 0..31, lanes >= 32 that of keys 32..63: both to both
             const auto r = __builtin_amdgcn_permlane32_swap(mine, mine, false, false);
             w.x = (uint32_t)r[0];
             w.y = (uint32_t)r[1];
         } else {
             w = lds_read_b64(maddr + slot * MASK_SLOT);
+            const bool last = (x == T - 1);
+            w.x &= last ? a.last_mask0 : 0xffffffffu;
+            w.y &= last ? a.last_mask1 : 0xffffffffu;
         }
-        const bool last = (x == T - 1);
-        w.x &= last ? a.last_mask0 : 0xffffffffu;
-        w.y &= last ? a.last_mask1 : 0xffffffffu;
         return w;
     };
     // ---- K/V tiles: async copies --------------------------------------------------------------
@@ -289,7 +304,6 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     // ================================ prologue: one memory round trip ================================
     // Requested at once, oldest first: q (this wave's 32 rows, staged through the second K/V stage,
     // which the prologue leaves unused, K-swizzled), then the mask words and K/V of tile 0.
-    const int qrow = qt * BM + wave * 32 + l32;
     {
         const int qbase = qt * BM + wave * 32 < N ? qt * BM + wave * 32 : N - 1;   // wave-uniform
         const uint16_t *qsrc = qb + (size_t)qbase * q_sn;

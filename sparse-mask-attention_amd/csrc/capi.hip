@@ -166,6 +166,7 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
     a.N = N;
     a.D = D;
     a.byte_mask = 0;
+    a.mask_out = nullptr;
     a.qtiles = (int)qtiles;
     split_scale(scale, &a.q_scale, &a.post_mul);
     last_tile_masks(N, &a.last_mask0, &a.last_mask1);
@@ -176,7 +177,8 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
 
 int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const uint8_t *mask,
                            int64_t mask_stride_b, int64_t mask_stride_h, void *out, float *lse,
-                           int B, int H, int N, int D, float scale, int dtype, void *stream)
+                           uint32_t *packed_out, int B, int H, int N, int D, float scale, int dtype,
+                           void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
     if (D != 32 && D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
@@ -190,7 +192,8 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
     // a lane's byte offset into the mask of one (b,h) is a 32-bit register
     if ((long long)N * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
-    if (misaligned(mask, 16) || (lse && misaligned(lse, 4))) return SMA_ERR_ALIGNMENT;
+    if (misaligned(mask, 16) || (lse && misaligned(lse, 4)) || (packed_out && misaligned(packed_out, 4)))
+        return SMA_ERR_ALIGNMENT;
     if (mask_stride_b < 0 || mask_stride_h < 0 || ((mask_stride_b | mask_stride_h) & 15)) return SMA_ERR_STRIDE;
 
     sma::AttnArgs a;
@@ -207,6 +210,7 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
     a.N = N;
     a.D = D;
     a.byte_mask = 1;
+    a.mask_out = packed_out;
     a.qtiles = (int)qtiles;
     split_scale(scale, &a.q_scale, &a.post_mul);
     last_tile_masks(N, &a.last_mask0, &a.last_mask1);

@@ -52,6 +52,7 @@ struct AttnArgs {
     int BH, H, N;
     int D;                          // head dim: 32, 64 or 128
     int byte_mask;                  // the mask is the caller's boolean tensor, not packed words
+    uint32_t *mask_out;             // byte_mask only: nullptr, or where to leave the packed words [Bm, Hm, N, nw]
     int qtiles;                     // ceil(N / 128): query tiles (work-groups) per (b,h)
     FastDiv div_qtiles, div_H;      // filled in by the launcher
     // exp(scale * s) is evaluated as exp2(post_mul * (q_scale * q) . k): q is multiplied by

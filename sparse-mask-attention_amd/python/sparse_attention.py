@@ -32,10 +32,11 @@ What differs from the reference, on purpose:
 * Head dims: the kernels exist for 64 (the reference's only one), 32 and 128.  Any other D <= 128
   is computed exactly by zero-padding q, k, v to the next of these (the scores and the first D output
   columns do not change; the scale stays 1/sqrt(D)) at the price of the padding copies.
-* ``sparse_attention_func`` (no autograd, the mask is used once) does not pack the mask: where the
-  kernel's limits allow (contiguous q, k, v, N a multiple of 16) one launch reads
-  the bool mask itself and forms the packed words tile by tile, which is 15-35 % faster than
-  pack + attention; otherwise it packs as the reference does.  Results are bit-identical.
+* The mask is not packed in a pass of its own: where the kernel's limits allow (contiguous q, k, v,
+  N a multiple of 16) one launch reads the bool mask itself and forms the packed words tile by
+  tile, which is 15-35 % faster than pack + attention; under autograd the same launch also leaves
+  the packed words behind for the backward.  Otherwise the mask is packed as the reference does.
+  Results are bit-identical either way.
 * ``.backward()`` works.  The reference calls a ``sparse_attn_cuda.backward`` that was never
   written (:91-94); here that function exists (two HIP kernels, dQ and dK/dV, from the saved
   log-sum-exp and the packed mask).  ``backward_recompute`` states the same gradients with PyTorch
@@ -100,7 +101,11 @@ def sparse_attention_ref(q, k, v, mask):
 # ----------------------------------------------------------------------------------------------
 
 class SparseAttentionFunction(Function):
-    """forward = fused HIP kernel (saves LSE); backward = the HIP dQ and dK/dV kernels."""
+    """forward = fused HIP kernel (saves LSE); backward = the HIP dQ and dK/dV kernels.
+
+    ``mask_packed`` may be None: the mask is then read as it is by the one-launch forward, which
+    leaves the packed words the backward needs as a by-product, or packed first where that kernel
+    does not apply."""
 
     @staticmethod
     def forward(ctx, q, k, v, mask_packed, mask_bool, scale, seq_len):
@@ -109,6 +114,16 @@ class SparseAttentionFunction(Function):
         q, k, v = _rows(q), _rows(k), _rows(v)
         out = torch.empty_like(q)
         lse = torch.empty(B, H, N, device=q.device, dtype=torch.float32)
+        if mask_packed is None:
+            mask_bool = _unexpand(mask_bool)
+            if sparse_attn_cuda.bool_mask_supported(q, k, v, mask_bool):
+                mask_packed = torch.empty(mask_bool.shape[0], mask_bool.shape[1], N, (N + 31) // 32,
+                                          device=q.device, dtype=torch.int32)
+                sparse_attn_cuda.forward_bool_mask(q, k, v, mask_bool, out, lse, scale, True, mask_packed)
+                ctx.save_for_backward(q, k, v, out, lse, mask_packed)
+                ctx.scale = scale
+                return out
+            mask_packed = pack_mask(mask_bool)
         sparse_attn_cuda.forward(q, k, v, mask_packed, out, lse, scale, True)
         ctx.save_for_backward(q, k, v, out, lse, mask_packed)
         ctx.scale = scale
@@ -173,8 +188,7 @@ def _unexpand(mask: torch.Tensor) -> torch.Tensor:
     return mask
 
 
-def _pack_shared(mask: torch.Tensor) -> torch.Tensor:
-    return pack_mask(_unexpand(mask))
+
 
 
 def _pad_head_dim(q, k, v):
@@ -211,8 +225,6 @@ def sparse_attention(q, k, v, mask, mask_packed=None):
     if orig_dtype == torch.float32:
         q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
 
-    if mask_packed is None:
-        mask_packed = _pack_shared(mask)
     q, k, v = _pad_head_dim(q, k, v)              # differentiable: the gradients are sliced back
     out = SparseAttentionFunction.apply(q, k, v, mask_packed, mask, scale, N)[..., :D]
 

@@ -56,7 +56,7 @@ def load():
         lib.sma_attn_bwd_strided.restype = ci
         lib.sma_attn_bwd_strided.argtypes = [tp] * 5 + [vp, vp, i64, i64, tp, tp, tp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_fwd_bool_mask.restype = ci
-        lib.sma_attn_fwd_bool_mask.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_attn_fwd_bool_mask.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         _lib = lib
     return _lib
 
@@ -154,9 +154,10 @@ def attn_bwd_strided(dout, q, k, v, out, lse, packed, grads=None, scale=None):
     return dq, dk, dv, delta
 
 
-def attn_fwd_bool_mask(q, k, v, mask, scale=None, want_lse=False, expect=SMA_OK):
+def attn_fwd_bool_mask(q, k, v, mask, scale=None, want_lse=False, expect=SMA_OK, want_packed=False):
     """Forward straight from the boolean mask ([1|B, 1|H, N, N], contiguous) through
-    sma_attn_fwd_bool_mask; returns out (and lse), or the status if `expect` is an error code."""
+    sma_attn_fwd_bool_mask; returns out (and lse) (and the packed words it leaves behind), or the
+    status if `expect` is an error code."""
     lib = load()
     B, H, N, D = q.shape
     if scale is None:
@@ -168,10 +169,13 @@ def attn_fwd_bool_mask(q, k, v, mask, scale=None, want_lse=False, expect=SMA_OK)
     msh = N * N if Hm == H and H > 1 else 0
     out = torch.full_like(q, float("nan"))
     lse = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device) if want_lse else None
+    packed = (torch.full((Bm, Hm, N, (N + 31) // 32), -1431655766, dtype=torch.int32, device=q.device)
+              if want_packed else None)
     st = lib.sma_attn_fwd_bool_mask(q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), msb, msh,
-                                    out.data_ptr(), lse.data_ptr() if want_lse else None, B, H, N, D, scale, dt,
-                                    _stream())
+                                    out.data_ptr(), lse.data_ptr() if want_lse else None,
+                                    packed.data_ptr() if want_packed else None, B, H, N, D, scale, dt, _stream())
     if expect != SMA_OK:
         return st
     assert st == SMA_OK, lib.sma_strerror(st)
-    return (out, lse) if want_lse else out
+    res = (out,) + ((lse,) if want_lse else ()) + ((packed,) if want_packed else ())
+    return res if len(res) > 1 else out

@@ -105,3 +105,21 @@ def test_limits_are_reported(dev):
     q, k, v, mask = _inputs(1, 1, 64, 96, torch.float16, 71)
     qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
     assert _capi.attn_fwd_bool_mask(qd, kd, vd, md, expect=_capi.SMA_ERR_HEAD_DIM) == _capi.SMA_ERR_HEAD_DIM
+
+
+@pytest.mark.parametrize("shape", ["BH", "11", "B1", "1H"])
+@pytest.mark.parametrize("N", [16, 80, 128, 400, 1008])
+def test_packed_words_are_left_behind(dev, N, shape):
+    """packed_out receives exactly what sma_pack_mask writes (every word, pad bits zero), so that a
+    backward can follow without a packing pass; shared masks are written once."""
+    B, H, D = 2, 3, 64
+    Bm, Hm = (1 if shape[0] == "1" else B), (1 if shape[1] == "1" else H)
+    q, k, v, _ = _inputs(B, H, N, D, torch.float16, 80 + N)
+    g = torch.Generator().manual_seed(N)
+    mask = torch.rand(Bm, Hm, N, N, generator=g) < 0.3
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    out, lse, packed = _capi.attn_fwd_bool_mask(qd, kd, vd, md, want_lse=True, want_packed=True)
+    torch.cuda.synchronize()
+    assert torch.equal(packed.cpu(), torch.from_numpy(O.pack_mask_ref(mask)))
+    want, want_lse = _capi.attn_fwd_strided(qd, kd, vd, packed, want_lse=True)
+    assert torch.equal(out, want) and torch.equal(lse, want_lse)

@@ -79,7 +79,7 @@ def test_argument_validation_needs_no_gpu(capi):
 
     def bcall(mask=p, msb=4096, msh=4096, **kw):
         a = dict(ok_args, **kw)
-        return fb(p, p, p, mask, msb, msh, p, None, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
+        return fb(p, p, p, mask, msb, msh, p, None, None, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
 
     assert bcall(D=96) == _capi.SMA_ERR_HEAD_DIM
     assert bcall(N=100) == _capi.SMA_ERR_BAD_SHAPE                            # not a multiple of 16
