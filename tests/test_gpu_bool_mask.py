@@ -123,3 +123,22 @@ def test_packed_words_are_left_behind(dev, N, shape):
     assert torch.equal(packed.cpu(), torch.from_numpy(O.pack_mask_ref(mask)))
     want, want_lse = _capi.attn_fwd_strided(qd, kd, vd, packed, want_lse=True)
     assert torch.equal(out, want) and torch.equal(lse, want_lse)
+
+
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C5"])
+def test_benchmark_workloads_at_full_size(dev, name):
+    """The BASELINE workloads whose length the kernel takes, whole: identical to pack + attention
+    (which the other files hold against the oracle at these sizes), words left behind identical to
+    the packer's, and the oracle-free property that V = 1 gives exactly 1 on every non-empty row."""
+    import harness
+    w = harness.WORKLOADS[name]
+    q, k, v, mask = harness.make_inputs(w, seed=42)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    packed = _capi.pack_mask(md)
+    want = _capi.attn_fwd(qd, kd, vd, packed)
+    got, words = _capi.attn_fwd_bool_mask(qd, kd, vd, md, want_packed=True)
+    assert torch.equal(got, want) and torch.equal(words, packed)
+    ones = _capi.attn_fwd_bool_mask(qd, kd, torch.ones_like(vd), md)
+    nonempty = md.any(dim=-1)
+    assert (ones[nonempty] == 1).all() and (ones[~nonempty] == 0).all()
+    torch.cuda.synchronize()
