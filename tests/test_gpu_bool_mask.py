@@ -142,3 +142,16 @@ def test_benchmark_workloads_at_full_size(dev, name):
     nonempty = md.any(dim=-1)
     assert (ones[nonempty] == 1).all() and (ones[~nonempty] == 0).all()
     torch.cuda.synchronize()
+
+
+def test_every_length_up_to_512(dev):
+    """All multiples of 16 up to 512 (every size of last tile, with and without a second word, one
+    to four work-groups per head), words included; one process, one launch pair per length."""
+    for N in range(16, 513, 16):
+        q, k, v, mask = _inputs(1, 2, N, 64, torch.float16, 5000 + N, keep=0.2)
+        qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+        packed = _capi.pack_mask(md)
+        got, words = _capi.attn_fwd_bool_mask(qd, kd, vd, md, want_packed=True)
+        assert torch.equal(words, packed), N
+        assert torch.equal(got, _capi.attn_fwd(qd, kd, vd, packed)), N
+    torch.cuda.synchronize()
