@@ -198,6 +198,51 @@ def test_forward_can_be_captured_in_a_graph_and_replayed(sa, dev):
         assert torch.equal(out_g, eager), f"replay {rep}"
 
 
+def test_training_step_can_be_captured_in_a_graph_and_replayed(sa, dev):
+    """Forward from the bool mask (packed words kept for the backward) and both backward kernels in
+    one captured graph; the only allocations are PyTorch's.  Each replay, on new values in the same
+    buffers and with eager work in between, must reproduce the eager step bit for bit."""
+    q, k, v, mask = _inputs(2, 2, 160, torch.float16, 22)
+    md = mask.to(dev)
+    leaves = [t.to(dev).requires_grad_(True) for t in (q, k, v)]
+    dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(5)).to(torch.float16).to(dev)
+
+    def step():
+        out = sa.sparse_attention(*leaves, md)
+        out.backward(dout)
+        return out
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            step()
+    torch.cuda.current_stream().wait_stream(side)
+    for t in leaves:
+        t.grad = None
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out_g = step()
+    grads_g = [t.grad for t in leaves]
+    for rep in range(3):
+        g = torch.Generator().manual_seed(200 + rep)
+        with torch.no_grad():
+            for t in leaves:
+                t.copy_(torch.randn(q.shape, generator=g).to(torch.float16))
+            md.copy_(torch.rand(mask.shape, generator=g) < 0.3)
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [out_g.clone()] + [x.clone() for x in grads_g]
+        eager_leaves = [t.detach().clone().requires_grad_(True) for t in leaves]
+        out_e = sa.sparse_attention(*eager_leaves, md)
+        out_e.backward(dout)
+        torch.cuda.synchronize()
+        want = [out_e] + [t.grad for t in eager_leaves]
+        for name, a, b in zip(("out", "dq", "dk", "dv"), got, want):
+            assert torch.equal(a, b), f"replay {rep}: {name}"
+
+
 @pytest.mark.parametrize("mshape", ["11", "B1", "BH"])
 def test_views_of_a_fused_projection_and_shared_masks_through_autograd(sa, dev, mshape):
     """q, k, v as slices of one [B, N, 3, H, D] projection output (no copies are made), the mask
