@@ -133,11 +133,13 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     const uint32_t q_rb = 2u * q_sn, k_rb = 2u * k_sn, v_rb = 2u * v_sn;                   // row pitch, bytes
 
     // ---- mask words: wave-private async copies, slot = tile % NSTAGE, lane i -> (row i/2, word i%2) ----
-    // BYTEMASK (N % 16 == 0): the wave's 32 x 64 bytes of a tile as two copies of 16 rows; lane i
+    // BYTEMASK (N >= 16): the wave's 32 x 64 bytes of a tile as two copies of 16 rows; lane i
     // fills (row 16j + i/4, position i%4) with the global 16-byte chunk position ^ ((row >> 2) & 3),
-    // which makes the reads below (lane = row, two chunks each) free of bank conflicts.  In a last
-    // tile of fewer than 64 keys the chunks beyond the row's end re-read its first chunk; their
-    // bits are cleared with the pad bits below.
+    // which makes the reads below (lane = row, two chunks each) free of bank conflicts.  The copies
+    // take any byte address (rows of N bytes start anywhere).  In a last tile of fewer than 64 keys
+    // every chunk that would reach beyond the row's end is read from the 16 bytes before that end
+    // instead, so that nothing after the mask's last byte is touched; the bits of the chunk that
+    // holds the end are shifted to their places below, those of later chunks cleared as pad bits.
     const int mrow = BYTEMASK ? 0 : qt * BM + wave * 32 + (lane >> 1);
     const uint32_t m_voff = BYTEMASK ? 0u : (uint32_t)(((size_t)(mrow < N ? mrow : N - 1) * nw + (lane & 1)) * 4);
     uint32_t mb_voff[2] = {0u, 0u}, mb_chunk[2] = {0u, 0u};
@@ -160,9 +162,16 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
             uint32_t vo[2] = {mb_voff[0], mb_voff[1]};
             if (ragged && x == T - 1) {
                 const uint32_t row_end = (uint32_t)(N - x * BN);       // bytes of the row left in this tile
+                // the lane offsets are unsigned: what is taken from them below is first taken from the
+                // base (a tile that is not the first has 64 bytes of the row before it; in the first,
+                // row_end = N >= 16 and nothing goes below zero)
+                const uint32_t back = x > 0 ? 16u : 0u;
+                src -= back;
 #pragma unroll
-                for (int j = 0; j < 2; ++j)
-                    if (mb_chunk[j] >= row_end) vo[j] -= mb_chunk[j];
+                for (int j = 0; j < 2; ++j) {
+                    vo[j] += back;
+                    if (mb_chunk[j] + 16 > row_end) vo[j] -= mb_chunk[j] + 16 - row_end;
+                }
             }
             async_copy_b128_at<OFF_MASK + SLOT * MASK_SLOT>(mask_dst, src, vo[0]);
             async_copy_b128_at<OFF_MASK + SLOT * MASK_SLOT + 1024>(mask_dst, src, vo[1]);
@@ -201,7 +210,14 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
             b2 = __builtin_amdgcn_udot4(d1.y, 0x80402010u, b2, false);
             b3 = __builtin_amdgcn_udot4(d1.w, 0x80402010u, b3, false);
             uint32_t mine = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
-            if (x == T - 1) mine &= hh ? a.last_mask1 : a.last_mask0;       // bits of keys >= N
+            if (x == T - 1) {
+                // the chunk that holds the row's end was copied from 16 bytes before that end: its
+                // bits move down to their places (zeros follow them)
+                const int row_end = N - x * BN, part = row_end >> 4, shift = (16 - (row_end & 15)) & 15;
+                const uint32_t lo = (mine & 0xffffu) >> (part == 2 * hh ? shift : 0);
+                const uint32_t hi = (mine >> 16) >> (part == 2 * hh + 1 ? shift : 0);
+                mine = (lo | (hi << 16)) & (hh ? a.last_mask1 : a.last_mask0);       // bits of keys >= N
+            }
             // a caller who will need the packed words (for the backward) gets them as a by-product
             if (words_out != nullptr && qrow < N && 2 * x + hh < nw) words_out[2 * x + hh] = mine;
             // lanes < 32 hold the word of keys 0..31, lanes >= 32 that of keys 32..63: both to both
@@ -589,7 +605,7 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     }
     if (a.byte_mask) {
         // built for contiguous rows only (checked by the C-ABI layer)
-        if (!packed || (a.N & 15) != 0) return hipErrorInvalidValue;
+        if (!packed || a.N < 16) return hipErrorInvalidValue;
         if (D == 32) { SMA_FWD_BYTEMASK_VARIANTS(32) } else if (D == 64) { SMA_FWD_BYTEMASK_VARIANTS(64) } else { SMA_FWD_BYTEMASK_VARIANTS(128) }
     } else if (D == 32) { SMA_FWD_VARIANTS(32) } else if (D == 64) { SMA_FWD_VARIANTS(64) } else { SMA_FWD_VARIANTS(128) }
 #undef SMA_FWD_VARIANTS

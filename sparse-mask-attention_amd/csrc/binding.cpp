@@ -106,20 +106,20 @@ void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor
 }
 
 // Limits of sma_attn_fwd_bool_mask, so that callers can choose between it and pack_mask + forward
-// without provoking an error: contiguous q, k, v, head dim 32, 64 or 128, N a multiple of 16, a
-// contiguous bool mask [1|B, 1|H, N, N] whose storage is 16-byte aligned.
+// without provoking an error: contiguous q, k, v, head dim 32, 64 or 128, 16 <= N < 46341, a
+// contiguous bool mask [1|B, 1|H, N, N].
 bool bool_mask_supported(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,
                          const torch::Tensor &mask)
 {
     if (!q.is_cuda() || q.dim() != 4 || mask.dim() != 4) return false;
     const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
-    if (!(D == 32 || D == 64 || D == 128) || N % 16 != 0 || N == 0 || N * N >= (int64_t(1) << 31)) return false;
+    if (!(D == 32 || D == 64 || D == 128) || N < 16 || N * N >= (int64_t(1) << 31)) return false;
     if (!q.is_contiguous() || !k.is_contiguous() || !v.is_contiguous()) return false;
     if (mask.scalar_type() != at::kBool || !mask.is_contiguous() || mask.device() != q.device()) return false;
     if (!((mask.size(0) == B || mask.size(0) == 1) && (mask.size(1) == H || mask.size(1) == 1) &&
           mask.size(2) == N && mask.size(3) == N))
         return false;
-    return reinterpret_cast<uintptr_t>(mask.data_ptr()) % 16 == 0;
+    return true;
 }
 
 void forward_bool_mask(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,
@@ -132,7 +132,7 @@ void forward_bool_mask(const torch::Tensor &q, const torch::Tensor &k, const tor
     const auto dt = q.scalar_type();
     TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "Unsupported dtype, need BF16 or FP16");
     TORCH_CHECK(bool_mask_supported(q, k, v, mask),
-                "forward_bool_mask needs contiguous q, k, v with head_dim 32, 64 or 128, N a multiple of 16 and a "
+                "forward_bool_mask needs contiguous q, k, v with head_dim 32, 64 or 128, N >= 16 and a "
                 "contiguous bool mask [B or 1, H or 1, N, N]; use pack_mask + forward otherwise");
     const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
     for (const torch::Tensor *t : {&k, &v, static_cast<const torch::Tensor *>(&out)}) {

@@ -187,14 +187,14 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
     const long long BH = (long long)B * H;
     if (BH == 0 || N == 0) return SMA_OK;
     if (!mask) return SMA_ERR_NULL_POINTER;
-    if (N % 16 != 0) return SMA_ERR_BAD_SHAPE;          // rows of the mask must start 16-byte aligned
+    if (N < 16) return SMA_ERR_BAD_SHAPE;               // a row holds at least one 16-byte copy
     const long long qtiles = (N + 127) / 128;
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
     // a lane's byte offset into the mask of one (b,h) is a 32-bit register
     if ((long long)N * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
-    if (misaligned(mask, 16) || (lse && misaligned(lse, 4)) || (packed_out && misaligned(packed_out, 4)))
+    if ((lse && misaligned(lse, 4)) || (packed_out && misaligned(packed_out, 4)))
         return SMA_ERR_ALIGNMENT;
-    if (mask_stride_b < 0 || mask_stride_h < 0 || ((mask_stride_b | mask_stride_h) & 15)) return SMA_ERR_STRIDE;
+    if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 
     sma::AttnArgs a;
     const sma_tensor t[4] = {dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D), dense(out, H, N, D)};

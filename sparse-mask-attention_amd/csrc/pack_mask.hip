@@ -9,12 +9,12 @@
 //                      (one global_load_dwordx4, fully coalesced), turns them into 16 bits, pairs up
 //                      with its neighbour lane, and even lanes store one word (coalesced 128 B per
 //                      wavefront).  Two independent spans per thread keep loads in flight.
-//   pack_row8_kernel   N % 8 == 0 (rows 8-byte aligned, e.g. N = 1000).  One wavefront per mask row:
-//                      lane l loads the 8 bytes at 8*l of a 512-byte segment (coalesced), makes 8
-//                      bits, the four lanes of a quad combine theirs with two DPP-style exchanges and
-//                      lane 4k stores word k of the segment; the last word of a row is short.
-//   pack_rows_kernel   any N.  One lane per output word, 4-byte loads when N % 4 == 0, byte loads
-//                      otherwise; the last word of a row is filled only up to column N-1.
+//   pack_row_kernel    any other N >= 8 (e.g. N = 1000) or mask address.  One wavefront per mask row:
+//                      lane l loads the 8 bytes at 8*l of a 512-byte segment (coalesced, at whatever
+//                      alignment the row has), makes 8 bits, the four lanes of a quad combine theirs
+//                      with two DPP-style exchanges and lane 4k stores word k of the segment.  The
+//                      lane that holds the row's end loads the row's last 8 bytes and shifts.
+//   pack_short_rows_kernel   N < 8: one lane per row, byte loads.
 //
 // A mask byte counts as "attend" when it is non-zero (torch.bool storage holds 0/1).
 //
@@ -73,28 +73,63 @@ __global__ __launch_bounds__(PACK_THREADS) void pack_flat_kernel(const u32x4 *__
 
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
-__global__ __launch_bounds__(PACK_THREADS) void pack_row8_kernel(const uint8_t *__restrict__ mask,
-                                                                 uint32_t *__restrict__ packed,
-                                                                 long long rows, int N, int nw)
+// U times eight bytes from any byte addresses, one global_load_dwordx2 each (gfx950 under ROCm
+// serves vector loads of any alignment; the compiler itself would split a load it cannot prove
+// aligned into bytes).  Issue and wait sit in one statement, so no use can come before the data.
+__device__ __forceinline__ void load8_any(u32x2 (&d)[1], const uint8_t *const (&p)[1])
+{
+    asm volatile("global_load_dwordx2 %0, %1, off\n\t"
+                 "s_waitcnt vmcnt(0)"
+                 : "=&v"(d[0]) : "v"(p[0]) : "memory");
+}
+__device__ __forceinline__ void load8_any(u32x2 (&d)[2], const uint8_t *const (&p)[2])
+{
+    asm volatile("global_load_dwordx2 %0, %2, off\n\t"
+                 "global_load_dwordx2 %1, %3, off\n\t"
+                 "s_waitcnt vmcnt(0)"
+                 : "=&v"(d[0]), "=&v"(d[1]) : "v"(p[0]), "v"(p[1]) : "memory");
+}
+__device__ __forceinline__ void load8_any(u32x2 (&d)[4], const uint8_t *const (&p)[4])
+{
+    asm volatile("global_load_dwordx2 %0, %4, off\n\t"
+                 "global_load_dwordx2 %1, %5, off\n\t"
+                 "global_load_dwordx2 %2, %6, off\n\t"
+                 "global_load_dwordx2 %3, %7, off\n\t"
+                 "s_waitcnt vmcnt(0)"
+                 : "=&v"(d[0]), "=&v"(d[1]), "=&v"(d[2]), "=&v"(d[3])
+                 : "v"(p[0]), "v"(p[1]), "v"(p[2]), "v"(p[3])
+                 : "memory");
+}
+
+// U: 512-byte segments in flight per wavefront (the host picks 1, 2 or 4 by the row length, so that
+// short rows do not issue loads that fetch nothing new)
+template <int U>
+__global__ __launch_bounds__(PACK_THREADS) void pack_row_kernel(const uint8_t *__restrict__ mask,
+                                                                uint32_t *__restrict__ packed,
+                                                                long long rows, int N, int nw)   // N >= 8
 {
     const int lane = threadIdx.x & 63;
     const long long row = (long long)blockIdx.x * (PACK_THREADS / 64) + (threadIdx.x >> 6);
     if (row >= rows) return;                       // whole wavefront leaves together
     const uint8_t *src = mask + row * (long long)N;
     uint32_t *dst = packed + row * (long long)nw;
-    for (int seg0 = 0; seg0 * 512 < N; seg0 += 4) {          // four 512-byte segments in flight
-        u32x2 d[4];
+    for (int seg0 = 0; seg0 * 512 < N; seg0 += U) {
+        u32x2 d[U];
+        const uint8_t *p[U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
+        for (int u = 0; u < U; ++u) {
             const int col = (seg0 + u) * 512 + lane * 8;    // first column of this lane's 8 bytes
-            u32x2 x = {0u, 0u};
-            if (col < N) x = *reinterpret_cast<const u32x2 *>(src + col);
-            d[u] = x;
+            // bytes that would lie beyond the row are not touched: the row's last 8 bytes instead
+            p[u] = src + (col + 8 <= N ? col : N - 8);
         }
+        load8_any(d, p);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            uint32_t b = __builtin_amdgcn_udot4(nonzero_bytes(d[u].x), 0x08040201u, 0u, false);
-            b = __builtin_amdgcn_udot4(nonzero_bytes(d[u].y), 0x80402010u, b, false);
+        for (int u = 0; u < U; ++u) {
+            const int col = (seg0 + u) * 512 + lane * 8;
+            uint64_t v = ((uint64_t)d[u].y << 32) | d[u].x;
+            if (col + 8 > N) v = col < N ? v >> (8 * (col + 8 - N)) : 0ull;      // the row's last columns, moved down
+            uint32_t b = __builtin_amdgcn_udot4(nonzero_bytes((uint32_t)v), 0x08040201u, 0u, false);
+            b = __builtin_amdgcn_udot4(nonzero_bytes((uint32_t)(v >> 32)), 0x80402010u, b, false);
             b <<= 8 * (lane & 3);                          // position inside the word of this quad
             b |= __shfl_xor(b, 1, 64);
             b |= __shfl_xor(b, 2, 64);
@@ -104,31 +139,16 @@ __global__ __launch_bounds__(PACK_THREADS) void pack_row8_kernel(const uint8_t *
     }
 }
 
-template <bool ALIGNED4>
-__global__ __launch_bounds__(PACK_THREADS) void pack_rows_kernel(const uint8_t *__restrict__ mask,
-                                                                 uint32_t *__restrict__ packed,
-                                                                 uint32_t total_words, int N, int nw)
+__global__ __launch_bounds__(PACK_THREADS) void pack_short_rows_kernel(const uint8_t *__restrict__ mask,
+                                                                       uint32_t *__restrict__ packed,
+                                                                       uint32_t rows, int N)            // N < 8
 {
-    const uint32_t idx = blockIdx.x * (uint32_t)PACK_THREADS + threadIdx.x;
-    if (idx >= total_words) return;
-    const uint32_t row = idx / (uint32_t)nw;
-    const int w = (int)(idx - row * (uint32_t)nw);
-    const uint8_t *src = mask + (size_t)row * N + 32 * w;
-    const int valid = min(32, N - 32 * w);          // columns of this word that exist (>= 1)
+    const uint32_t row = blockIdx.x * (uint32_t)PACK_THREADS + threadIdx.x;
+    if (row >= rows) return;
+    const uint8_t *src = mask + (size_t)row * N;
     uint32_t acc = 0u;
-    if (ALIGNED4) {
-        // N % 4 == 0: the row start and every 4-column group are 4-byte aligned and a group is
-        // either wholly inside the row or wholly outside.
-#pragma unroll
-        for (int g = 0; g < 8; ++g) {
-            uint32_t x = 0u;
-            if (4 * g < valid) x = *reinterpret_cast<const uint32_t *>(src + 4 * g);
-            acc |= __builtin_amdgcn_udot4(nonzero_bytes(x), 0x08040201u, 0u, false) << (4 * g);
-        }
-    } else {
-        for (int j = 0; j < valid; ++j) acc |= (uint32_t)(src[j] != 0) << j;
-    }
-    packed[idx] = acc;
+    for (int j = 0; j < N; ++j) acc |= (uint32_t)(src[j] != 0) << j;
+    packed[row] = acc;
 }
 
 }  // namespace
@@ -145,19 +165,15 @@ hipError_t launch_pack_mask(const uint8_t *mask, uint32_t *packed, long long row
         const unsigned grid = (unsigned)((n_chunks + per_block - 1) / per_block);
         hipLaunchKernelGGL(pack_flat_kernel, dim3(grid), dim3(PACK_THREADS), 0, stream,
                            reinterpret_cast<const u32x4 *>(mask), packed, n_chunks);
-    } else if ((N % 8 == 0) && ((reinterpret_cast<uintptr_t>(mask) & 7u) == 0)) {
+    } else if (N >= 8) {
         const unsigned grid = (unsigned)((rows + PACK_THREADS / 64 - 1) / (PACK_THREADS / 64));
-        hipLaunchKernelGGL(pack_row8_kernel, dim3(grid), dim3(PACK_THREADS), 0, stream, mask, packed, rows, N, nw);
+        const int segments = (N + 511) / 512;
+        auto kernel = segments >= 4 ? pack_row_kernel<4> : segments >= 2 ? pack_row_kernel<2> : pack_row_kernel<1>;
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(PACK_THREADS), 0, stream, mask, packed, rows, N, nw);
     } else {
-        const uint32_t total = (uint32_t)(rows * nw);
-        const unsigned grid = (total + PACK_THREADS - 1) / PACK_THREADS;
-        const bool aligned4 = (N % 4 == 0) && ((reinterpret_cast<uintptr_t>(mask) & 3u) == 0);
-        if (aligned4)
-            hipLaunchKernelGGL(pack_rows_kernel<true>, dim3(grid), dim3(PACK_THREADS), 0, stream,
-                               mask, packed, total, N, nw);
-        else
-            hipLaunchKernelGGL(pack_rows_kernel<false>, dim3(grid), dim3(PACK_THREADS), 0, stream,
-                               mask, packed, total, N, nw);
+        const unsigned grid = (unsigned)((rows + PACK_THREADS - 1) / PACK_THREADS);
+        hipLaunchKernelGGL(pack_short_rows_kernel, dim3(grid), dim3(PACK_THREADS), 0, stream, mask, packed,
+                           (uint32_t)rows, N);
     }
     return hipGetLastError();
 }

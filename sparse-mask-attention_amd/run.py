@@ -46,7 +46,7 @@ def sparse_attention_hip_two_launches(q, k, v, mask):
 
 def sparse_attention_hip_fwd(q, k, v, mask):
     """Boolean mask in, output out: allocation + the forward that reads the boolean mask itself
-    where it applies (N a multiple of 16), else the two launches above."""
+    where it applies (contiguous q, k, v, N >= 16), else the two launches above."""
     import sparse_attn_cuda as ext
     if not ext.bool_mask_supported(q, k, v, mask):
         return sparse_attention_hip_two_launches(q, k, v, mask)

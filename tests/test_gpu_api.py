@@ -322,7 +322,7 @@ def test_backward_from_an_expanded_gradient(sa, dev):
 
 def test_expanded_mask_is_packed_once(sa, dev, monkeypatch):
     """mask.expand(B, H, N, N) (zero strides) must reach the packer with the extents it really has."""
-    B, H, N = 3, 4, 100                            # not a multiple of 16: the packing path
+    B, H, N = 3, 4, 12                             # shorter than 16: the packing path
     q, k, v, _ = _inputs(B, H, N, torch.float16, 14)
     g = torch.Generator().manual_seed(15)
     small = (torch.rand(1, 1, N, N, generator=g) < 0.3).to(dev)
@@ -362,9 +362,14 @@ def test_inference_entry_point_reads_the_bool_mask_itself(sa, dev, monkeypatch):
     ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask[:1, :1].expand(2, 3, 192, 192))
     assert torch.allclose(shared.float().cpu(), ref, atol=1e-2, rtol=1e-2)
     calls.clear()
-    q, k, v, mask = _inputs(1, 2, 100, torch.float16, 17)                                   # N % 16 != 0
+    q, k, v, mask = _inputs(1, 2, 101, torch.float16, 17)                                   # rows at odd addresses
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    odd = sa.sparse_attention_func(qd, kd, vd, md)
+    assert calls == [] and torch.equal(odd, sa.sparse_attention_func(qd, kd, vd, None, mask_packed=real(md)))
+    calls.clear()
+    q, k, v, mask = _inputs(1, 2, 12, torch.float16, 17)                                    # N < 16
     sa.sparse_attention_func(q.to(dev), k.to(dev), v.to(dev), mask.to(dev))
-    assert calls == [(1, 2, 100, 100)]
+    assert calls == [(1, 2, 12, 12)]
     # fp32 inputs: computed in bf16 through the same path, returned as fp32
     q, k, v, mask = _inputs(1, 2, 128, torch.float32, 18)
     o32 = sa.sparse_attention_func(q.to(dev), k.to(dev), v.to(dev), mask.to(dev))

@@ -22,7 +22,7 @@ def _inputs(B, H, N, D, dtype, seed, keep=0.25):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("D", [32, 64, 128])
-@pytest.mark.parametrize("N", [16, 48, 64, 80, 128, 144, 192, 256, 400, 512, 1008, 1024])
+@pytest.mark.parametrize("N", [16, 17, 48, 64, 65, 79, 80, 100, 128, 144, 192, 250, 256, 400, 511, 512, 1000, 1001, 1008, 1024])
 def test_equals_pack_then_attention(dev, dtype, D, N):
     B, H = 2, 3
     q, k, v, mask = _inputs(B, H, N, D, dtype, 300 + N + D)
@@ -99,7 +99,7 @@ def test_scales_many_heads_and_long_rows(dev):
 
 
 def test_limits_are_reported(dev):
-    q, k, v, mask = _inputs(1, 1, 104, 64, torch.float16, 70)                  # rows not 16-byte aligned
+    q, k, v, mask = _inputs(1, 1, 15, 64, torch.float16, 70)                   # a row shorter than one 16-byte copy
     qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
     assert _capi.attn_fwd_bool_mask(qd, kd, vd, md, expect=_capi.SMA_ERR_BAD_SHAPE) == _capi.SMA_ERR_BAD_SHAPE
     q, k, v, mask = _inputs(1, 1, 64, 96, torch.float16, 71)
@@ -107,8 +107,27 @@ def test_limits_are_reported(dev):
     assert _capi.attn_fwd_bool_mask(qd, kd, vd, md, expect=_capi.SMA_ERR_HEAD_DIM) == _capi.SMA_ERR_HEAD_DIM
 
 
+@pytest.mark.parametrize("offset", [1, 2, 4, 8, 13])
+def test_mask_at_any_byte_address(dev, offset):
+    """The mask need not start on a 16-byte boundary, and it may end with its allocation's last
+    byte: no copy reaches beyond it (every 16-byte copy that would is moved back)."""
+    B, H, N, D = 2, 2, 200, 64
+    q, k, v, mask = _inputs(B, H, N, D, torch.float16, 600 + offset)
+    qd, kd, vd = (t.to(dev) for t in (q, k, v))
+    buf = torch.ones(offset + mask.numel(), dtype=torch.bool, device=dev)
+    md = buf[offset:].view(B, H, N, N)
+    md.copy_(mask)
+    assert md.data_ptr() % 16 == offset % 16 and md.is_contiguous()
+    packed = _capi.pack_mask(md)
+    assert torch.equal(packed.cpu(), torch.from_numpy(O.pack_mask_ref(mask)))
+    got, lse, words = _capi.attn_fwd_bool_mask(qd, kd, vd, md, want_lse=True, want_packed=True)
+    want, want_lse = _capi.attn_fwd(qd, kd, vd, packed, want_lse=True)
+    torch.cuda.synchronize()
+    assert torch.equal(words, packed) and torch.equal(got, want) and torch.equal(lse, want_lse)
+
+
 @pytest.mark.parametrize("shape", ["BH", "11", "B1", "1H"])
-@pytest.mark.parametrize("N", [16, 80, 128, 400, 1008])
+@pytest.mark.parametrize("N", [16, 35, 80, 128, 250, 400, 1001, 1008])
 def test_packed_words_are_left_behind(dev, N, shape):
     """packed_out receives exactly what sma_pack_mask writes (every word, pad bits zero), so that a
     backward can follow without a packing pass; shared masks are written once."""
@@ -125,9 +144,9 @@ def test_packed_words_are_left_behind(dev, N, shape):
     assert torch.equal(out, want) and torch.equal(lse, want_lse)
 
 
-@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C5"])
+@pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
 def test_benchmark_workloads_at_full_size(dev, name):
-    """The BASELINE workloads whose length the kernel takes, whole: identical to pack + attention
+    """The BASELINE workloads, whole: identical to pack + attention
     (which the other files hold against the oracle at these sizes), words left behind identical to
     the packer's, and the oracle-free property that V = 1 gives exactly 1 on every non-empty row."""
     import harness
@@ -145,13 +164,16 @@ def test_benchmark_workloads_at_full_size(dev, name):
 
 
 def test_every_length_up_to_512(dev):
-    """All multiples of 16 up to 512 (every size of last tile, with and without a second word, one
-    to four work-groups per head), words included; one process, one launch pair per length."""
-    for N in range(16, 513, 16):
+    """All lengths from 16 to 512 (every size and alignment of last tile and of the rows' first
+    bytes, with and without a second word, one to four work-groups per head), words included; one
+    process, one launch pair per length."""
+    for N in range(16, 513):
         q, k, v, mask = _inputs(1, 2, N, 64, torch.float16, 5000 + N, keep=0.2)
         qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
         packed = _capi.pack_mask(md)
         got, words = _capi.attn_fwd_bool_mask(qd, kd, vd, md, want_packed=True)
         assert torch.equal(words, packed), N
         assert torch.equal(got, _capi.attn_fwd(qd, kd, vd, packed)), N
+        if N % 37 == 0:
+            assert torch.equal(packed.cpu(), torch.from_numpy(O.pack_mask_ref(mask))), N
     torch.cuda.synchronize()

@@ -56,6 +56,20 @@ def test_nonzero_bytes_count_as_true(dev):
         assert np.array_equal(got.cpu().numpy(), O.pack_mask_ref(raw.numpy() != 0))
 
 
+def test_every_length_at_several_alignments(dev):
+    """Rows of every length up to 140 bytes (and some long odd ones) starting 0, 1 and 5 bytes into
+    an allocation that ends with the mask's last byte: every alignment of every row."""
+    g = torch.Generator().manual_seed(8)
+    for N in list(range(1, 141)) + [255, 511, 513, 999, 1001, 1031]:
+        m = torch.rand(1, 2, N, N, generator=g) > 0.6
+        want = O.pack_mask_ref(m)
+        for off in (0, 1, 5):
+            buf = torch.ones(off + m.numel(), dtype=torch.bool, device=dev)
+            view = buf[off:].view(1, 2, N, N)
+            view.copy_(m)
+            assert np.array_equal(_capi.pack_mask(view).cpu().numpy(), want), (N, off)
+
+
 def test_unaligned_base_pointer(dev):
     # a mask that starts 1 byte into an allocation takes the general (row) kernel
     g = torch.Generator().manual_seed(6)

@@ -82,10 +82,10 @@ def test_argument_validation_needs_no_gpu(capi):
         return fb(p, p, p, mask, msb, msh, p, None, None, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
 
     assert bcall(D=96) == _capi.SMA_ERR_HEAD_DIM
-    assert bcall(N=100) == _capi.SMA_ERR_BAD_SHAPE                            # not a multiple of 16
+    assert bcall(N=12) == _capi.SMA_ERR_BAD_SHAPE                             # shorter than one 16-byte copy
+    assert bcall(N=46341) == _capi.SMA_ERR_BAD_SHAPE                          # N * N does not fit 31 bits
     assert bcall(mask=None) == _capi.SMA_ERR_NULL_POINTER
-    assert bcall(mask=ctypes.c_void_p(0x1004)) == _capi.SMA_ERR_ALIGNMENT
-    assert bcall(msh=24) == _capi.SMA_ERR_STRIDE
+    assert bcall(msh=-24) == _capi.SMA_ERR_STRIDE
     assert bcall(dtype=5) == _capi.SMA_ERR_DTYPE
     assert bcall(B=0) == _capi.SMA_OK
 
