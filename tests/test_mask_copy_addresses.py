@@ -1,0 +1,57 @@
+"""CPU check of the address arithmetic of the forward that reads the boolean mask
+(csrc/attn_fwd.hip, issue_mask / mask_words): restated here with numpy for every lane of every wave,
+so that for every sequence length
+  * each lane offset is a non-negative 32-bit number (the hardware adds it unsigned to the base),
+  * each 16-byte copy lies inside the N*N bytes of its (b,h) mask (nothing before the first or
+    after the last byte is read),
+  * the chunk a lane converts holds the 16 columns it stands for, or, for the chunk that contains
+    the row's end, those columns after the right shift the kernel applies.
+A GPU cannot tell the second point (an over-read of a few bytes usually lands in mapped memory)."""
+import numpy as np
+import pytest
+
+BM, BN = 128, 64
+
+
+def _check(N):
+    T = (N + BN - 1) // BN
+    ragged = N % BN != 0
+    qtiles = (N + BM - 1) // BM
+    lane = np.arange(64)
+    for qt in {0, qtiles - 1}:
+        for wave in range(4):
+            for x in {0, T - 2, T - 1} & set(range(T)):
+                base = x * BN
+                for j in range(2):
+                    row = 16 * j + (lane >> 2)
+                    grow = qt * BM + wave * 32 + row
+                    grow = np.where(grow < N, grow, N - 1).astype(np.int64)
+                    chunk = ((lane & 3) ^ ((row >> 2) & 3)) << 4
+                    voff = grow * N + chunk
+                    src = base
+                    row_end = N - x * BN
+                    if ragged and x == T - 1:
+                        back = 16 if x > 0 else 0
+                        src -= back
+                        voff = voff + back
+                        voff = np.where(chunk + 16 > row_end, voff - (chunk + 16 - row_end), voff)
+                    assert src >= 0 and (voff >= 0).all() and (voff < 2**32).all(), (N, x)
+                    addr = src + voff
+                    assert (addr >= 0).all() and (addr + 16 <= N * N).all(), (N, x)
+                    col0 = addr - grow * N                      # first column the copy holds
+                    want0 = x * BN + chunk
+                    whole = want0 + 16 <= N
+                    assert (col0[whole] == want0[whole]).all(), (N, x)
+                    part = (want0 < N) & ~whole                 # the chunk that holds the row's end
+                    shift = (16 - (row_end & 15)) & 15
+                    assert ((chunk[part] >> 4) == (row_end >> 4)).all() and (col0[part] + shift == want0[part]).all(), (N, x)
+
+
+def test_every_length_up_to_1100():
+    for N in range(16, 1101):
+        _check(N)
+
+
+@pytest.mark.parametrize("N", [2047, 4095, 8191, 46340])
+def test_long_rows(N):
+    _check(N)
