@@ -14,6 +14,8 @@
 //                      alignment the row has), makes 8 bits, the four lanes of a quad combine theirs
 //                      with two DPP-style exchanges and lane 4k stores word k of the segment.  The
 //                      lane that holds the row's end loads the row's last 8 bytes and shifts.
+//   pack_few_lanes_per_row_kernel   the same for rows of 8 to 256 bytes with 4, 8, 16 or 32 lanes per
+//                      row: a wavefront packs 16 to 2 rows at once.
 //   pack_short_rows_kernel   N < 8: one lane per row, byte loads.
 //
 // A mask byte counts as "attend" when it is non-zero (torch.bool storage holds 0/1).
@@ -139,6 +141,34 @@ __global__ __launch_bounds__(PACK_THREADS) void pack_row_kernel(const uint8_t *_
     }
 }
 
+// Rows of 8 to 256 bytes: 2^lpr_shift = 4, 8, 16 or 32 lanes per row, so a wavefront packs 16 to 2
+// rows at once instead of leaving most of its lanes idle.
+__global__ __launch_bounds__(PACK_THREADS) void pack_few_lanes_per_row_kernel(const uint8_t *__restrict__ mask,
+                                                                              uint32_t *__restrict__ packed,
+                                                                              long long rows, int N, int nw,
+                                                                              int lpr_shift)
+{
+    const int lane = threadIdx.x & 63;
+    const long long wave = (long long)blockIdx.x * (PACK_THREADS / 64) + (threadIdx.x >> 6);
+    const long long row = (wave << (6 - lpr_shift)) + (lane >> lpr_shift);
+    if ((wave << (6 - lpr_shift)) >= rows) return;            // whole wavefront leaves together
+    const bool live = row < rows;
+    const long long r = live ? row : rows - 1;
+    const int l = lane & ((1 << lpr_shift) - 1);
+    const int col = l * 8;
+    u32x2 d[1];
+    const uint8_t *const p[1] = {mask + r * (long long)N + (col + 8 <= N ? col : N - 8)};
+    load8_any(d, p);
+    uint64_t v = ((uint64_t)d[0].y << 32) | d[0].x;
+    if (col + 8 > N) v = col < N ? v >> (8 * (col + 8 - N)) : 0ull;
+    uint32_t b = __builtin_amdgcn_udot4(nonzero_bytes((uint32_t)v), 0x08040201u, 0u, false);
+    b = __builtin_amdgcn_udot4(nonzero_bytes((uint32_t)(v >> 32)), 0x80402010u, b, false);
+    b <<= 8 * (lane & 3);
+    b |= __shfl_xor(b, 1, 64);
+    b |= __shfl_xor(b, 2, 64);
+    if (live && (lane & 3) == 0 && (l >> 2) < nw) packed[r * (long long)nw + (l >> 2)] = b;
+}
+
 __global__ __launch_bounds__(PACK_THREADS) void pack_short_rows_kernel(const uint8_t *__restrict__ mask,
                                                                        uint32_t *__restrict__ packed,
                                                                        uint32_t rows, int N)            // N < 8
@@ -165,6 +195,13 @@ hipError_t launch_pack_mask(const uint8_t *mask, uint32_t *packed, long long row
         const unsigned grid = (unsigned)((n_chunks + per_block - 1) / per_block);
         hipLaunchKernelGGL(pack_flat_kernel, dim3(grid), dim3(PACK_THREADS), 0, stream,
                            reinterpret_cast<const u32x4 *>(mask), packed, n_chunks);
+    } else if (N >= 8 && N <= 256) {
+        int lpr_shift = 2;                                     // lanes per row: 8 bytes each, at least a quad
+        while ((8 << lpr_shift) < N) ++lpr_shift;
+        const long long waves = (rows + (64 >> lpr_shift) - 1) >> (6 - lpr_shift);
+        const unsigned grid = (unsigned)((waves + PACK_THREADS / 64 - 1) / (PACK_THREADS / 64));
+        hipLaunchKernelGGL(pack_few_lanes_per_row_kernel, dim3(grid), dim3(PACK_THREADS), 0, stream, mask, packed,
+                           rows, N, nw, lpr_shift);
     } else if (N >= 8) {
         const unsigned grid = (unsigned)((rows + PACK_THREADS / 64 - 1) / (PACK_THREADS / 64));
         const int segments = (N + 511) / 512;
