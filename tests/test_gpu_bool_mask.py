@@ -177,3 +177,31 @@ def test_every_length_up_to_512(dev):
         if N % 37 == 0:
             assert torch.equal(packed.cpu(), torch.from_numpy(O.pack_mask_ref(mask))), N
     torch.cuda.synchronize()
+
+
+def test_mask_larger_than_4_GiB(dev):
+    """Ten (b,h) masks of 21000 x 21000 bytes: 4.41 GB, so the offsets of the later ones need more than
+    32 bits (those inside one mask stay below 2^31).  Identical to pack + attention everywhere; rows
+    of the first and the last (b,h) against a float32 formulation with PyTorch ops on the device."""
+    B, H, N, D = 2, 5, 21000, 64
+    g = torch.Generator(device=dev).manual_seed(77)
+    qd, kd, vd = [torch.randn(B, H, N, D, generator=g, device=dev).half() for _ in range(3)]
+    md = torch.empty(B, H, N, N, dtype=torch.bool, device=dev)
+    for b in range(B):
+        for h in range(H):
+            md[b, h] = torch.rand(N, N, generator=g, device=dev) < 0.05
+    assert md.numel() > 2**32
+    md[1, 4, N - 1, :] = False
+    packed = _capi.pack_mask(md)
+    want = _capi.attn_fwd(qd, kd, vd, packed)
+    got, words = _capi.attn_fwd_bool_mask(qd, kd, vd, md, want_packed=True)
+    torch.cuda.synchronize()
+    assert torch.equal(words, packed) and torch.equal(got, want)
+    rows = torch.tensor([0, 1, 127, 128, 10000, N - 2, N - 1], device=dev)
+    for b, h in ((0, 0), (1, 4)):
+        s = (qd[b, h, rows].float() @ kd[b, h].float().T) / math.sqrt(D)
+        s = s.masked_fill(~md[b, h, rows], -math.inf)
+        p = torch.softmax(s, dim=-1).nan_to_num(0.0)
+        ref = p @ vd[b, h].float()
+        assert torch.allclose(got[b, h, rows].float(), ref, atol=1e-2, rtol=1e-2), (b, h)
+    assert (got[1, 4, N - 1] == 0).all()
