@@ -136,7 +136,8 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     // BYTEMASK (N >= 16): the wave's 32 x 64 bytes of a tile as two copies of 16 rows; lane i
     // fills (row 16j + i/4, position i%4) with the global 16-byte chunk position ^ ((row >> 2) & 3),
     // which makes the reads below (lane = row, two chunks each) free of bank conflicts.  The copies
-    // take any byte address (rows of N bytes start anywhere).  In a last tile of fewer than 64 keys
+    // take any byte address (rows of N bytes start anywhere; ROCm runs the memory pipeline in its
+    // unaligned access mode, in which a 16-byte copy may start at any byte).  In a last tile of fewer than 64 keys
     // every chunk that would reach beyond the row's end is read from the 16 bytes before that end
     // instead, so that nothing after the mask's last byte is touched; the bits of the chunk that
     // holds the end are shifted to their places below, those of later chunks cleared as pad bits.
