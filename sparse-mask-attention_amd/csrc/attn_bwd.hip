@@ -16,10 +16,14 @@
 //                        initial value), dS^T packed to 16 bit is the B operand of dQ^T += K^T dS^T
 //                        (K^T by transposing LDS reads).  Also writes delta to the workspace.
 //   attn_bwd_dkv_kernel  one work-group = 128 keys (lane = key), walks the query tiles:
-//                        S = Q K^T and dP = dO V^T with K, V fragments held in registers; lse and
-//                        delta of the tile's rows come from LDS (broadcast reads), the mask bit of
-//                        (row, key) is bit (key % 32) of the row's word; P and dS packed to 16 bit
-//                        are the B operands of dV^T += dO^T P and dK^T += Q^T dS.
+//                        S = Q K^T and dP = dO V^T with K, V fragments held in registers; -lse and
+//                        -delta of the tile's rows are read from LDS (broadcast reads) straight
+//                        into the accumulators as their initial values, so the products leave
+//                        s - lse and dP - delta; the mask bit of (row, key) is bit (key % 32) of the
+//                        row's word; P and dS packed to 16 bit are the B operands of
+//                        dV^T += dO^T P and dK^T += Q^T dS.  The loop over the query tiles is
+//                        unrolled by the two ring stages, so every LDS address in it is a
+//                        register plus an immediate.
 //
 // Tiles (64 rows x 64 x 16 bit) are copied global -> LDS by global_load_lds_dwordx4 into two
 // stages, one tile ahead; the 16-byte chunks of a row are XOR-swizzled with bitrev3((row >> 1) & 7),
@@ -308,7 +312,7 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_bwd_dq_ker
 // ------------------------------------------------------------------------------------------------
 // DK / DV: which of the two gradients this instance produces (both for head dim 64; one per launch
 // for head dim 128, where both sets of accumulators do not fit the register file).
-template <bool BF16, int HDIM, bool DK, bool DV>
+template <bool BF16, int HDIM, bool DK, bool DV, bool POSTMUL>
 __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwdArgs a)
 {
     using E = Elem<BF16>;
@@ -331,7 +335,8 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     const int N = a.N, nw = (N + 31) >> 5;
     const int T = (N + BN - 1) / BN;
     const bool ragged = (N & (BN - 1)) != 0;
-    const float pm = a.post_mul;
+    const float pm = POSTMUL ? a.post_mul : 1.0f;
+    const float lse_mul = -LOG2E / pm;                // pm is a power of two: exact
 
     const int bi = (int)fastdiv((uint32_t)bh, a.div_H), hi = bh - bi * a.H;
     const uint16_t *qb = slab(a.q, bi, hi), *dob = slab(a.dout, bi, hi);
@@ -345,6 +350,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     const int key = key0 + l32;
     const int kr = key < N ? key : N - 1;
     const uint32_t key_ok = key < N ? 0xffffffffu : 0u;
+    const uint32_t key_w = key < N ? 1u : 0u;         // width of the bit field that holds this key's mask bit
     const int wi = (key0 >> 5) < nw ? (key0 >> 5) : nw - 1;     // this wave's mask word of a row
     u32x4 kf[KS], vf[DK ? KS : 1];
 #pragma unroll
@@ -385,22 +391,31 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
             if constexpr (DV) dvacc[b][i] = 0.f;
         }
 
-    for (int t = 0; t < T; ++t) {
-        const int st = t & 1;
+    // one q tile; the ring stage is a compile-time constant so that every LDS address of the body is
+    // a register plus an immediate
+    auto tile = [&](int t, auto st_c) __attribute__((always_inline)) {
+        constexpr int st = decltype(st_c)::value;
         const uint32_t so = lds0 + st * STAGE_BYTES;
         const uint32_t aux = lds0 + OFF_AUX + st * AUX_BYTES;
         WAIT_VMCNT(0);
         if (wave == 0) {
-            // lse of the tile's rows -> log2 units; rows that kept nothing or lie beyond N -> +inf
+            // lse of the tile's rows -> what the score accumulators start from, -lse * log2(e) / pm, so
+            // that exp2(pm * accumulator) is the probability; rows that kept nothing or lie beyond N
+            // -> -inf (probability 0)
             const uint32_t p = aux + 1024 + lane * 4;
             const float l = *(LDS_PTR(float))(uintptr_t)p;
             const bool dead = (t * BN + lane >= N) || (l == -__builtin_inff());
-            *(LDS_PTR(float))(uintptr_t)p = dead ? __builtin_inff() : l * LOG2E;
+            *(LDS_PTR(float))(uintptr_t)p = dead ? -__builtin_inff() : l * lse_mul;
+        }
+        if (wave == 1) {
+            // -delta: the dP accumulators start from it
+            const uint32_t p = aux + 1280 + lane * 4;
+            *(LDS_PTR(float))(uintptr_t)p = -*(LDS_PTR(float))(uintptr_t)p;
         }
         if (ragged && t == T - 1) zero_tile_tail(so, 2 * NH, t * BN, N, tc, wave, lane);
         __syncthreads();
         if (t + 1 < T) issue(t + 1, st ^ 1);
-        if (!wave_valid) continue;
+        if (!wave_valid) return;
 
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
@@ -415,9 +430,20 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
             }
             if (__builtin_amdgcn_ballot_w64((((any >> l32) & 1u) & key_ok) != 0u) == 0ull) continue;
 
+            // the accumulators start from the rows' -lse (scaled) and -delta, read straight into them:
+            // the products then leave s - lse and dP - delta, with no subtraction per element
             f32x16 sacc, dacc;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) { sacc[i] = 0.f; dacc[i] = 0.f; }
+            for (int g = 0; g < 4; ++g) {
+                const u32x4 Lr = lds_read_b128(aux + 1024 + rsel + 32 * g);
+                u32x4 Dr = {0u, 0u, 0u, 0u};
+                if constexpr (DK) Dr = lds_read_b128(aux + 1280 + rsel + 32 * g);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    sacc[4 * g + j] = __builtin_bit_cast(float, (uint32_t)Lr[j]);
+                    dacc[4 * g + j] = __builtin_bit_cast(float, (uint32_t)Dr[j]);
+                }
+            }
 #pragma unroll
             for (int s = 0; s < KS; ++s)
                 sacc = E::mfma(lds_read_b128(tr.rowaddr[s & 3] + so + (s >> 2) * TILE_BYTES + 4096 * blk), kf[s], sacc);
@@ -431,18 +457,13 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
             uint32_t pp[2][4] = {}, ps[2][4] = {};       // the one a single-gradient instance leaves unused is dropped
 #pragma unroll
             for (int g = 0; g < 4; ++g) {
-                const u32x4 Lr = lds_read_b128(aux + 1024 + rsel + 32 * g);
-                u32x4 Dr = {0u, 0u, 0u, 0u};
-                if constexpr (DK) Dr = lds_read_b128(aux + 1280 + rsel + 32 * g);
                 float p[4], d[4];
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)mw[g][j], (uint32_t)l32, 1u) & key_ok;
-                    const float Lj = __builtin_bit_cast(float, (uint32_t)Lr[j]);
-                    const float Dj = __builtin_bit_cast(float, (uint32_t)Dr[j]);
-                    const float e = __builtin_amdgcn_exp2f(__builtin_fmaf(sacc[4 * g + j], pm, -Lj));
+                    const uint32_t keep = (uint32_t)__builtin_amdgcn_sbfe((int)mw[g][j], (uint32_t)l32, key_w);
+                    const float e = __builtin_amdgcn_exp2f(POSTMUL ? sacc[4 * g + j] * pm : sacc[4 * g + j]);
                     p[j] = __builtin_bit_cast(float, __builtin_bit_cast(uint32_t, e) & keep);
-                    d[j] = p[j] * (dacc[4 * g + j] - Dj);
+                    d[j] = p[j] * dacc[4 * g + j];
                 }
                 // elements 4g .. 4g+3 are pairs (2i, 2i+1) with i = 2(g & 1), 2(g & 1) + 1 of u = g >> 1
                 if constexpr (DV) {
@@ -477,6 +498,10 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
                 }
             }
         }
+    };
+    for (int t = 0; t < T; t += 2) {
+        tile(t, std::integral_constant<int, 0>{});
+        if (t + 1 < T) tile(t + 1, std::integral_constant<int, 1>{});
     }
     WAIT_VMCNT(0);
     __syncthreads();
@@ -500,6 +525,16 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
     }
 }
 
+// Launches the dK/dV instance for (dtype, head dim, gradients) with or without the post-multiplier.
+template <bool BF16, int HDIM, bool DK, bool DV>
+void launch_dkv(bool postmul, dim3 grid, dim3 block, hipStream_t stream, const AttnBwdArgs &a)
+{
+    if (postmul)
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<BF16, HDIM, DK, DV, true>), grid, block, 0, stream, a);
+    else
+        hipLaunchKernelGGL((attn_bwd_dkv_kernel<BF16, HDIM, DK, DV, false>), grid, block, 0, stream, a);
+}
+
 }  // namespace
 
 hipError_t launch_attn_bwd(const AttnBwdArgs &args, bool bf16, hipStream_t stream)
@@ -510,32 +545,33 @@ hipError_t launch_attn_bwd(const AttnBwdArgs &args, bool bf16, hipStream_t strea
     const long long groups = (long long)a.BH * a.qtiles;
     if (groups == 0) return hipSuccess;
     const dim3 grid((unsigned)groups), block(NTHREADS);
+    const bool postmul = a.post_mul != 1.0f;       // exp2(pm * s) needs its multiplication only then
     // dQ first: it also fills the delta workspace that the dK/dV kernel reads (same stream).
     if (a.D == 2 * HD) {
         if (bf16) {
             hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 128>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 128, true, false>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 128, false, true>), grid, block, 0, stream, a);
+            launch_dkv<true, 128, true, false>(postmul, grid, block, stream, a);
+            launch_dkv<true, 128, false, true>(postmul, grid, block, stream, a);
         } else {
             hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 128>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 128, true, false>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 128, false, true>), grid, block, 0, stream, a);
+            launch_dkv<false, 128, true, false>(postmul, grid, block, stream, a);
+            launch_dkv<false, 128, false, true>(postmul, grid, block, stream, a);
         }
     } else if (a.D == HD) {
         if (bf16) {
             hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 64>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 64, true, true>), grid, block, 0, stream, a);
+            launch_dkv<true, 64, true, true>(postmul, grid, block, stream, a);
         } else {
             hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 64>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 64, true, true>), grid, block, 0, stream, a);
+            launch_dkv<false, 64, true, true>(postmul, grid, block, stream, a);
         }
     } else {
         if (bf16) {
             hipLaunchKernelGGL((attn_bwd_dq_kernel<true, 32>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<true, 32, true, true>), grid, block, 0, stream, a);
+            launch_dkv<true, 32, true, true>(postmul, grid, block, stream, a);
         } else {
             hipLaunchKernelGGL((attn_bwd_dq_kernel<false, 32>), grid, block, 0, stream, a);
-            hipLaunchKernelGGL((attn_bwd_dkv_kernel<false, 32, true, true>), grid, block, 0, stream, a);
+            launch_dkv<false, 32, true, true>(postmul, grid, block, stream, a);
         }
     }
     return hipGetLastError();
