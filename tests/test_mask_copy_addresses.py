@@ -1,4 +1,5 @@
-"""CPU check of the address arithmetic of the forward that reads the boolean mask
+"""CPU checks of address arithmetic that a GPU run cannot judge (an over-read of a few bytes usually
+lands in mapped memory).  First, the forward that reads the boolean mask
 (csrc/attn_fwd.hip, issue_mask / mask_words): restated here with numpy for every lane of every wave,
 so that for every sequence length
   * each lane offset is a non-negative 32-bit number (the hardware adds it unsigned to the base),
@@ -55,3 +56,40 @@ def test_every_length_up_to_1100():
 @pytest.mark.parametrize("N", [2047, 4095, 8191, 46340])
 def test_long_rows(N):
     _check(N)
+
+
+def _check_packer_row(N, lanes_per_row=64):
+    """csrc/pack_mask.hip, pack_row_kernel / pack_few_lanes_per_row_kernel: lane l of a segment takes
+    the 8 bytes at column 8l, or the row's last 8 bytes shifted down when those would cross the
+    row's end; restated with numpy on one row of distinct bits."""
+    rng = np.random.default_rng(N)
+    row = rng.integers(0, 2, N).astype(np.uint8)
+    nw = (N + 31) // 32
+    words = np.zeros(nw, dtype=np.uint64)
+    seg_bytes = 8 * lanes_per_row
+    for seg in range((N + seg_bytes - 1) // seg_bytes):
+        for lane in range(lanes_per_row):
+            col = seg * seg_bytes + lane * 8
+            start = col if col + 8 <= N else N - 8
+            assert 0 <= start and start + 8 <= N, (N, col)           # the load stays inside the row
+            v = int.from_bytes(row[start:start + 8].tobytes(), "little")
+            if col + 8 > N:
+                v = v >> (8 * (col + 8 - N)) if col < N else 0
+            bits = sum(((v >> (8 * i)) & 1) << i for i in range(8))
+            w = col // 32
+            if w < nw:
+                words[w] |= np.uint64(bits << (8 * (lane & 3)))
+    want = np.zeros(nw, dtype=np.uint64)
+    for c in range(N):
+        want[c // 32] |= np.uint64(int(row[c]) << (c % 32))
+    assert (words == want).all(), N
+
+
+def test_packer_row_loads_stay_inside_the_row_and_place_every_bit():
+    for N in list(range(8, 600)) + [999, 1000, 1001, 1023, 1025, 2047]:
+        _check_packer_row(N)
+    for N in range(8, 257):                                  # the kernel with fewer lanes per row
+        lanes = 4
+        while 8 * lanes < N:
+            lanes *= 2
+        _check_packer_row(N, lanes)
