@@ -7,7 +7,7 @@ so that for every sequence length
     after the last byte is read),
   * the chunk a lane converts holds the 16 columns it stands for, or, for the chunk that contains
     the row's end, those columns after the right shift the kernel applies.
-A GPU cannot tell the second point (an over-read of a few bytes usually lands in mapped memory)."""
+Second, the packer's row loads (csrc/pack_mask.hip), further down."""
 import numpy as np
 import pytest
 
