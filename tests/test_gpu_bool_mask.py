@@ -146,7 +146,7 @@ def test_packed_words_are_left_behind(dev, N, shape):
 
 @pytest.mark.parametrize("name", ["C1", "C2", "C3", "C4", "C5"])
 def test_benchmark_workloads_at_full_size(dev, name):
-    """The BASELINE workloads, whole: identical to pack + attention
+    """The five benchmark workloads, whole: identical to pack + attention
     (which the other files hold against the oracle at these sizes), words left behind identical to
     the packer's, and the oracle-free property that V = 1 gives exactly 1 on every non-empty row."""
     import harness
