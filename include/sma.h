@@ -28,6 +28,7 @@ extern "C" {
 #define SMA_ERR_LAUNCH        -6   /* the HIP runtime refused the launch (hipGetLastError) */
 #define SMA_ERR_ALIGNMENT     -7   /* q/k/v/out not 16-byte aligned, or mask_packed/lse not 4-byte aligned */
 #define SMA_ERR_STRIDE        -8   /* a stride is negative, not a multiple of 8 elements, or too large */
+#define SMA_ERR_WORKSPACE     -9   /* B*H*N exceeds SMA_STATIC_WS_ROWS (sma_attn_bwd_static_ws only) */
 
 #define SMA_DTYPE_F16   0
 #define SMA_DTYPE_BF16  1
@@ -94,6 +95,24 @@ int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *ma
 int sma_attn_bwd(const void *dout, const void *q, const void *k, const void *v, const void *out,
                  const float *lse, const uint32_t *mask_packed, void *dq, void *dk, void *dv,
                  float *delta_ws, int B, int H, int N, int D, float scale, int dtype, void *stream);
+
+/* sma_attn_bwd without the workspace argument, for callers that cannot allocate device memory at
+ * all (code running under HIP graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc): the per-row sums that the two kernels exchange live in a fixed array inside the
+ * library's device image (SMA_STATIC_WS_ROWS floats = 4 MiB, held by every GPU the library has
+ * been called on until the process ends).  Arguments and results are exactly those of
+ * sma_attn_bwd.  The call allocates nothing; B*H*N > SMA_STATIC_WS_ROWS returns SMA_ERR_WORKSPACE
+ * and launches nothing.  All calls on one GPU share the array: calls that may overlap in time (on
+ * different streams of the same GPU) race and must use sma_attn_bwd with workspaces of their own.
+ * The first call on a device looks the array's address up (hipGetSymbolAddress); make that call
+ * outside graph capture.
+ *
+ * No counterpart in the reference: this entry point exists only for callers that cannot allocate.
+ */
+#define SMA_STATIC_WS_ROWS (1 << 20)
+int sma_attn_bwd_static_ws(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                           const float *lse, const uint32_t *mask_packed, void *dq, void *dk, void *dv,
+                           int B, int H, int N, int D, float scale, int dtype, void *stream);
 
 /* A [B,H,N,D] tensor of 16-bit elements with explicit strides, in ELEMENTS.  The D elements of a
  * row are contiguous (stride 1, not stored).  Every stride must be >= 0 and a multiple of 8 (rows

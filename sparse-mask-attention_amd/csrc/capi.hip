@@ -1,6 +1,8 @@
 // extern "C" layer of libsma_hip.so: argument validation and dispatch.  See include/sma.h.
 #include <math.h>
 
+#include <atomic>
+
 #include "sma.h"
 #include "sma_internal.h"
 
@@ -29,6 +31,29 @@ int to_rows(const sma_tensor *t, int N, int D, sma::Rows *r)
     return SMA_OK;
 }
 
+// Workspace of sma_attn_bwd_static_ws: the per-row sums the two backward kernels exchange, held in
+// the library's own device image instead of a caller's buffer.  Every GPU the library runs on has
+// its own copy at its own address; the name below is only a host-side handle for
+// hipGetSymbolAddress and is never passed to a kernel.
+constexpr long long STATIC_WS_ROWS = 1ll << 20;          // B*H*N the entry point accepts (4 MiB)
+static __device__ __align__(256) float scratch[STATIC_WS_ROWS];
+
+// Device address of `scratch` on the current device, looked up once per device ordinal.
+float *static_workspace()
+{
+    static std::atomic<float *> cached[64];     // nullptr = not asked yet; racing threads store the same address
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+    float *p = cached[dev].load(std::memory_order_acquire);
+    if (p == nullptr) {
+        void *sym = nullptr;
+        if (hipGetSymbolAddress(&sym, HIP_SYMBOL(scratch)) != hipSuccess || sym == nullptr) return nullptr;
+        p = static_cast<float *>(sym);
+        cached[dev].store(p, std::memory_order_release);
+    }
+    return p;
+}
+
 }  // namespace
 
 extern "C" {
@@ -47,6 +72,7 @@ const char *sma_strerror(int code)
     case SMA_ERR_LAUNCH:       return "HIP kernel launch failed";
     case SMA_ERR_ALIGNMENT:    return "misaligned pointer";
     case SMA_ERR_STRIDE:       return "bad stride: negative, not a multiple of 8 elements, or too large";
+    case SMA_ERR_WORKSPACE:    return "problem too large for the library's static workspace";
     default:                   return "unknown error code";
     }
 }
@@ -228,6 +254,19 @@ int sma_attn_bwd(const void *dout, const void *q, const void *k, const void *v, 
     const int64_t msh = (int64_t)N * ((N + 31) / 32);
     return sma_attn_bwd_strided(&t[0], &t[1], &t[2], &t[3], &t[4], lse, mask_packed, msh * H, msh,
                                 &t[5], &t[6], &t[7], delta_ws, B, H, N, D, scale, dtype, stream);
+}
+
+int sma_attn_bwd_static_ws(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                           const float *lse, const uint32_t *mask_packed, void *dq, void *dk, void *dv,
+                           int B, int H, int N, int D, float scale, int dtype, void *stream)
+{
+    if (B < 0 || H < 0 || N < 0) return SMA_ERR_BAD_SHAPE;
+    if ((long long)B * H * N > STATIC_WS_ROWS) return SMA_ERR_WORKSPACE;
+    float *ws = static_workspace();
+    if (ws == nullptr) return SMA_ERR_LAUNCH;
+    // Both kernels run on `stream`, the first writes every entry the second reads: nothing has to
+    // be cleared between calls, and what a previous (larger) call left behind is never read.
+    return sma_attn_bwd(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, ws, B, H, N, D, scale, dtype, stream);
 }
 
 int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *mask_packed,

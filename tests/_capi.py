@@ -16,6 +16,8 @@ SMA_ERR_SCALE = -5
 SMA_ERR_LAUNCH = -6
 SMA_ERR_ALIGNMENT = -7
 SMA_ERR_STRIDE = -8
+SMA_ERR_WORKSPACE = -9
+SMA_STATIC_WS_ROWS = 1 << 20
 SMA_DTYPE_F16 = 0
 SMA_DTYPE_BF16 = 1
 
@@ -50,6 +52,8 @@ def load():
         lib.sma_attn_fwd.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_bwd.restype = ci
         lib.sma_attn_bwd.argtypes = [vp] * 11 + [ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_attn_bwd_static_ws.restype = ci
+        lib.sma_attn_bwd_static_ws.argtypes = [vp] * 10 + [ci, ci, ci, ci, cf, ci, vp]
         tp, i64 = ctypes.POINTER(SmaTensor), ctypes.c_int64
         lib.sma_attn_fwd_strided.restype = ci
         lib.sma_attn_fwd_strided.argtypes = [tp, tp, tp, vp, i64, i64, tp, vp, ci, ci, ci, ci, cf, ci, vp]
@@ -106,6 +110,24 @@ def attn_bwd(dout, q, k, v, out, lse, packed, scale=None):
                           delta.data_ptr(), B, H, N, D, scale, dt, _stream())
     assert st == SMA_OK, lib.sma_strerror(st)
     return dq, dk, dv, delta
+
+
+def attn_bwd_static_ws(dout, q, k, v, out, lse, packed, scale=None, expect=SMA_OK):
+    """Backward through sma_attn_bwd_static_ws (no workspace argument); returns (dq, dk, dv), or the
+    status if `expect` is an error code.  Outputs are poisoned first."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    dq, dk, dv = (torch.full_like(q, float("nan")) for _ in range(3))
+    st = lib.sma_attn_bwd_static_ws(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                                    lse.data_ptr(), packed.data_ptr(), dq.data_ptr(), dk.data_ptr(),
+                                    dv.data_ptr(), B, H, N, D, scale, dt, _stream())
+    if expect != SMA_OK:
+        return st
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return dq, dk, dv
 
 
 def _mask_strides(packed, B, H):
