@@ -52,6 +52,31 @@ const char *sma_strerror(int code);
  */
 int sma_pack_mask(const uint8_t *mask, uint32_t *packed, int B, int H, int N, void *stream);
 
+/* Tile map of a packed mask: which 64-key tiles matter to which block of 64 query rows.
+ *
+ *   tile_map  uint32 [B,H,T,2,TW], T = ceil(N/64) blocks of 64 query rows (and as many key tiles of
+ *             64 keys), TW = ceil(T/32) words: for row block r, word group 0 holds one bit per key
+ *             tile t (bit t%32 of word t/32) that is set when some mask bit of the 64 x 64 block
+ *             (r, t) is set; word group 1 one bit that is set when every bit of the block is set
+ *             (rows and columns below N).  sma_tile_map_words(N) = T*2*TW words per (batch entry,
+ *             head).  Every word is written.
+ *
+ * sma_attn_fwd_map visits only the key tiles whose first bit is set: for the others nothing is
+ * copied and nothing computed, which is what a block-structured mask (sliding window, block-sparse,
+ * causal) needs; the reference's own skip (csrc/sparse_attention.cu:238-252) still loads the tile
+ * (:211) and is taken per 64 query rows.  A map costs one pass over the packed words; make it once
+ * for a mask that is used many times.  N <= 131072.
+ *
+ * sma_pack_mask_map = sma_pack_mask followed by sma_tile_map on its output (tile_map may be NULL:
+ * then it is sma_pack_mask).
+ *
+ * No counterpart in the reference beyond the block skip cited above.
+ */
+long long sma_tile_map_words(int N);
+int sma_tile_map(const uint32_t *mask_packed, uint32_t *tile_map, int B, int H, int N, void *stream);
+int sma_pack_mask_map(const uint8_t *mask, uint32_t *packed, uint32_t *tile_map, int B, int H, int N,
+                      void *stream);
+
 /* Fused masked attention forward:  out = softmax_row(mask ? (q k^T) * scale : -inf) v.
  *
  *   q, k, v      [B,H,N,D] fp16 or bf16 (dtype), D = 64 (the reference's only head dim), 32 or 128
@@ -72,6 +97,14 @@ int sma_pack_mask(const uint8_t *mask, uint32_t *packed, int B, int H, int N, vo
 int sma_attn_fwd(const void *q, const void *k, const void *v, const uint32_t *mask_packed,
                  void *out, float *lse, int B, int H, int N, int D, float scale, int dtype,
                  void *stream);
+
+/* sma_attn_fwd with a tile map (see sma_tile_map) of the same packed mask; tile_map == NULL is
+ * sma_attn_fwd.  The results are those of sma_attn_fwd bit for bit; only the tiles visited differ.
+ * A map that does not belong to the mask gives wrong results (tiles it calls empty are not read).
+ */
+int sma_attn_fwd_map(const void *q, const void *k, const void *v, const uint32_t *mask_packed,
+                     const uint32_t *tile_map, void *out, float *lse, int B, int H, int N, int D,
+                     float scale, int dtype, void *stream);
 
 /* Masked attention backward:  given dout = dLoss/dout, the gradients with respect to q, k and v.
  *
@@ -142,6 +175,14 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
                          const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
                          const sma_tensor *out, float *lse, int B, int H, int N, int D, float scale,
                          int dtype, void *stream);
+
+/* sma_attn_fwd_strided with a tile map: contiguous [Bm,Hm,T,2,TW] with the mask's own Bm, Hm (1
+ * where the mask stride is 0), or NULL.
+ */
+int sma_attn_fwd_map_strided(const sma_tensor *q, const sma_tensor *k, const sma_tensor *v,
+                             const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                             const uint32_t *tile_map, const sma_tensor *out, float *lse, int B, int H,
+                             int N, int D, float scale, int dtype, void *stream);
 
 /* sma_pack_mask and sma_attn_fwd in one launch, for a mask that is used once: the kernel reads the
  * boolean bytes themselves and forms the packed words of each 64-key tile on the fly, so the packing

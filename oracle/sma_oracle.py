@@ -16,6 +16,11 @@ Functions and the reference lines they follow (paths under the reference tree):
                             for tiny inputs only (an independent second statement).
 * ``unpack_mask_ref``       inverse, reading side ``csrc/sparse_attention.cu:284``
                             (``(word >> (col % 32)) & 1``).
+* ``tile_map_ref``          which 64-key tiles hold a set mask bit for which block of 64 query rows, and
+                            which hold nothing else: the block-level emptiness test of
+                            ``csrc/sparse_attention.cu:238-252`` (there per 64 query rows, after the
+                            tile has been loaded) stated over the whole mask; ``tile_map_loops`` is
+                            the literal loop over blocks and entries, for tiny inputs.
 * ``sparse_attention_ref``  the six ops of ``python/sparse_attention.py:29-42`` (twin:
                             ``run.py:158-165``): matmul, * 1/sqrt(D), masked_fill(~mask,-inf),
                             softmax, nan_to_num(nan=0), matmul.  Tests call it in fp32 on
@@ -31,7 +36,10 @@ Pins (see tests/test_oracle.py): the pack format is pinned by ``numpy.packbits``
 closed forms: all-True mask equals dense softmax attention, a one-hot mask row returns
 exactly that value row, an empty mask row returns zeros, q = 0 returns the mean of the
 kept value rows, joint key permutation invariance, row independence, and the float64
-brute force.  ``lse_ref`` is pinned by ``scipy.special.logsumexp`` on the kept scores.
+brute force.  ``tile_map_ref`` is pinned by the literal loops, by known answers (all-True: every
+tile live and full; all-False: nothing; a single True entry: one live bit, nothing full; a ragged
+last tile is full when its valid entries are all True) and by the invariant that masking out every
+tile it calls empty changes nothing.  ``lse_ref`` is pinned by ``scipy.special.logsumexp`` on the kept scores.
 The reference ships no golden vectors for this path, so none are checked here.
 """
 from __future__ import annotations
@@ -45,6 +53,57 @@ import torch
 # ---------------------------------------------------------------------------
 # mask packing
 # ---------------------------------------------------------------------------
+
+def tile_map_shape(N: int):
+    """(blocks of 64 query rows, 2, words of 32 key tiles of 64 keys) per (batch entry, head)."""
+    T = (N + 63) // 64
+    return (T, 2, (T + 31) // 32)
+
+
+def tile_map_ref(mask) -> np.ndarray:
+    """uint32 ``[B,H,T,2,TW]``: bit t%32 of word t//32 of group 0 says that the 64 x 64 block (row
+    block, key tile t) of the mask holds a True entry, of group 1 that it holds nothing but True entries
+    (only rows and columns below N exist).  Bits of tiles that do not exist are zero."""
+    m = _as_numpy_bool(mask)
+    B, H, N, _ = m.shape
+    QT, _, TW = tile_map_shape(N)
+    T = (N + 63) // 64
+    some = np.zeros((B, H, QT * 64, T * 64), dtype=bool)
+    some[:, :, :N, :N] = m
+    hole = np.zeros((B, H, QT * 64, T * 64), dtype=bool)
+    hole[:, :, :N, :N] = ~m
+    some = some.reshape(B, H, QT, 64, T, 64).any(axis=(3, 5))
+    full = ~hole.reshape(B, H, QT, 64, T, 64).any(axis=(3, 5))
+    out = np.zeros((B, H, QT, 2, TW * 32), dtype=bool)
+    out[:, :, :, 0, :T] = some
+    out[:, :, :, 1, :T] = full
+    bits = np.packbits(out, axis=-1, bitorder="little")
+    return np.ascontiguousarray(bits).view("<u4").reshape(B, H, QT, 2, TW)
+
+
+def tile_map_loops(mask) -> np.ndarray:
+    """The same as ``tile_map_ref`` as literal loops over blocks and their entries (tiny inputs)."""
+    m = _as_numpy_bool(mask)
+    B, H, N, _ = m.shape
+    QT, _, TW = tile_map_shape(N)
+    out = np.zeros((B, H, QT, 2, TW), dtype=np.uint32)
+    for b in range(B):
+        for h in range(H):
+            for qt in range(QT):
+                for t in range((N + 63) // 64):
+                    any_set, all_set = False, True
+                    for i in range(64 * qt, min(N, 64 * qt + 64)):
+                        for j in range(64 * t, min(N, 64 * t + 64)):
+                            if m[b, h, i, j]:
+                                any_set = True
+                            else:
+                                all_set = False
+                    if any_set:
+                        out[b, h, qt, 0, t // 32] |= np.uint32(1 << (t % 32))
+                    if all_set:
+                        out[b, h, qt, 1, t // 32] |= np.uint32(1 << (t % 32))
+    return out
+
 
 def n_words(N: int) -> int:
     """Words per mask row: ``csrc/sparse_attention.cu:555``."""

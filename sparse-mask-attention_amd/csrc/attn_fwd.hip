@@ -33,8 +33,12 @@
 //   reference r = the online softmax does not track the exact running maximum.  r moves (and O, l
 //                 are rescaled) only when a row's scores leave the window [r-8, r+8] upwards, or
 //                 when its first finite score lies below the window; probabilities stay <= 2^8.
-//   skipping    = a wavefront whose own 32 x 64 block of mask bits is empty skips its GEMMs and its
-//                 softmax for that tile (the tile itself is still copied, see the main loop).
+//   skipping    = with a tile map (one "some bit set" and one "all bits set" bit per 128 x 64 block
+//                 of the mask, made by the packer) the work-group visits only the key tiles that
+//                 hold a set bit for its rows: no copies, no barrier for the others; a block whose
+//                 bits are all set needs no mask words and no bias.  Without a map every tile is
+//                 copied.  Either way a wavefront whose own 32 x 64 block of mask bits is empty
+//                 skips its GEMMs and its softmax for that tile.
 //   head dim    = the description above is for 64.  128 runs the same code on two column halves of
 //                 64 (see Cfg below): twice the MFMAs per tile for the same softmax work, a ring of
 //                 two stages and two work-groups per CU.  32 uses half of every tile row.
@@ -121,6 +125,23 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     const float pm = POSTMUL ? a.post_mul : 1.0f;
 
     const int bi = (int)fastdiv((uint32_t)bh, a.div_H), hi = bh - bi * a.H;
+    // ---- tile map: which key tiles hold a set mask bit for this work-group's rows ("live"; the map
+    // also says which hold nothing else, which this kernel does not use).  The map has one row of
+    // bits (one per key tile, 32 per word) for every block of 64 query rows: this work-group ORs
+    // the rows of its two blocks.  The first words are requested here with scalar loads and awaited
+    // just before the first copies are issued; the address arithmetic in between covers the latency.
+    const int TW = (T + 31) >> 5;
+    const uint32_t *mapw = nullptr, *mapw2 = nullptr;       // the two 64-row blocks (the same one if the second does not exist)
+    if constexpr (!BYTEMASK) {
+        if (a.tile_map != nullptr) {
+            mapw = a.tile_map + bi * a.map_sb + hi * a.map_sh + (size_t)(2 * qt) * 2 * TW;
+            mapw2 = (2 * qt + 1 < T) ? mapw + 2 * TW : mapw;
+        }
+    }
+    uint32_t live_w = 0xffffffffu, live_w2 = 0u;
+    if (mapw != nullptr)
+        asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0"
+                     : "=&s"(live_w), "=&s"(live_w2) : "s"(mapw), "s"(mapw2) : "memory");
     const uint16_t *qb = slab(a.q, bi, hi);
     const uint16_t *kb = slab(a.k, bi, hi);
     const uint16_t *vb = slab(a.v, bi, hi);
@@ -202,15 +223,19 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
             // this lane: the 32 bytes of row l32 for keys 32hh .. 32hh+31 -> one word
             const u32x4 d0 = lds_read_b128(maddr + slot * MASK_SLOT + (((2 * hh) ^ msw) << 4));
             const u32x4 d1 = lds_read_b128(maddr + slot * MASK_SLOT + (((2 * hh + 1) ^ msw) << 4));
-            uint32_t b0 = __builtin_amdgcn_udot4(d0.x, 0x08040201u, 0u, false);
-            uint32_t b1 = __builtin_amdgcn_udot4(d0.z, 0x08040201u, 0u, false);
-            uint32_t b2 = __builtin_amdgcn_udot4(d1.x, 0x08040201u, 0u, false);
-            uint32_t b3 = __builtin_amdgcn_udot4(d1.z, 0x08040201u, 0u, false);
-            b0 = __builtin_amdgcn_udot4(d0.y, 0x80402010u, b0, false);
-            b1 = __builtin_amdgcn_udot4(d0.w, 0x80402010u, b1, false);
-            b2 = __builtin_amdgcn_udot4(d1.y, 0x80402010u, b2, false);
-            b3 = __builtin_amdgcn_udot4(d1.w, 0x80402010u, b3, false);
-            uint32_t mine = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            // a byte counts as "attend" when it is non-zero, as in the packer: nz() leaves 0x80 in
+            // every non-zero byte, the dot products weigh those with 1, 2, 4 .. 128 (times 128)
+            auto nz = [](uint32_t x) -> uint32_t { return (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u; };
+            uint32_t b0 = __builtin_amdgcn_udot4(nz(d0.x), 0x08040201u, 0u, false);
+            uint32_t b1 = __builtin_amdgcn_udot4(nz(d0.z), 0x08040201u, 0u, false);
+            uint32_t b2 = __builtin_amdgcn_udot4(nz(d1.x), 0x08040201u, 0u, false);
+            uint32_t b3 = __builtin_amdgcn_udot4(nz(d1.z), 0x08040201u, 0u, false);
+            b0 = __builtin_amdgcn_udot4(nz(d0.y), 0x80402010u, b0, false);
+            b1 = __builtin_amdgcn_udot4(nz(d0.w), 0x80402010u, b1, false);
+            b2 = __builtin_amdgcn_udot4(nz(d1.y), 0x80402010u, b2, false);
+            b3 = __builtin_amdgcn_udot4(nz(d1.w), 0x80402010u, b3, false);
+            // each partial value is 128 x (8 bits): bits 7..14
+            uint32_t mine = (b0 >> 7) | (b1 << 1) | (b2 << 9) | (b3 << 17);
             if (x == T - 1) {
                 // the chunk that holds the row's end was copied from 16 bytes before that end: its
                 // bits move down to their places (zeros follow them)
@@ -337,14 +362,41 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         }
     }
     using std::integral_constant;
-    issue_mask(0, integral_constant<int, 0>{});
-    issue_kv(0, integral_constant<int, 0>{});
+    // the map word has had the whole address arithmetic above to arrive
+    if (mapw != nullptr) asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(live_w), "+s"(live_w2) :: "memory");
+    live_w |= live_w2;
+    if ((T & 31) != 0 && TW == 1) live_w &= (1u << (T & 31)) - 1u;
+    const int n_visits = TW == 1 ? __builtin_popcount(live_w) : T;
+    // Walk over the set bits of the "live" words: `live_w` holds the bits of word `cur_w` that have
+    // not been visited yet.  Words beyond the first (N > 2048) are fetched when the walk gets there.
+    int cur_w = 0;
+    auto next_tile = [&]() __attribute__((always_inline)) -> int {     // next live tile, T if there is none; wave-uniform
+        while (live_w == 0u) {
+            if (++cur_w >= TW) return T;
+            uint32_t lv = 0xffffffffu, lv2 = 0u;
+            if (mapw != nullptr)
+                asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0\n\ts_waitcnt lgkmcnt(0)"
+                             : "=&s"(lv), "=&s"(lv2) : "s"(mapw + cur_w), "s"(mapw2 + cur_w) : "memory");
+            lv |= lv2;
+            if (cur_w == TW - 1 && (T & 31) != 0) lv &= (1u << (T & 31)) - 1u;
+            live_w = lv;
+        }
+        const int b = __builtin_ctz(live_w);
+        live_w &= live_w - 1u;
+        return 32 * cur_w + b;
+    };
+    const int t_first = next_tile();
+    if (t_first < T) {
+        issue_mask(t_first, integral_constant<int, 0>{});
+        issue_kv(t_first, integral_constant<int, 0>{});
+    }
     // small LDS table for the mask: entry n (16 B) holds four floats, float j = (bit j of n) ? 0 : -inf
     if (tid < 64)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
     const bool even_progress = NH == 1 && (int)blockIdx.x >= a.tail_start;   // three work-groups per CU
-    if (even_progress && T >= 4) __builtin_amdgcn_s_setprio(3);
-    wait_vmcnt<C::COPIES>();          // q has landed; the copies of tile 0 may still be in flight
+    if (even_progress && n_visits >= 4) __builtin_amdgcn_s_setprio(3);
+    if (t_first < T) wait_vmcnt<C::COPIES>();     // q has landed; the copies of the first tile may still be in flight
+    else wait_vmcnt<0>();
     // ---- Q^T as MFMA B operands, scaled by scale*log2(e)/post_mul:
     //      lane holds query row l32, d = 16*s + 8*hh .. +7
     u32x4 qf[KS];
@@ -483,40 +535,44 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     };
 
     // ================================ main loop ================================
-    // Tile t uses stage and mask slot t % 2; the loop is unrolled by 2 so that these are constants.
-    // In iteration t:
-    //   wait for the copies of tile t  ->  barrier  ->  request the copies of tile t + 1 (mask
-    //   words, then K/V) into the stage the barrier has freed  ->  compute, unless this wave's
-    //   32 x 64 block of mask bits is empty.
+    // The tiles visited: every tile whose "some bit set" bit is on (all of them without a map), in
+    // ascending order; the prologue has requested the first.  The i-th visit uses stage and mask
+    // slot i % 2; the loop is unrolled by 2 so that these are constants.
+    // In a visit of tile t:
+    //   wait for the copies of tile t  ->  barrier  ->  request the copies of the next tile to be
+    //   visited (mask words, then K/V) into the stage the barrier has freed  ->  compute, unless
+    //   this wave's 32 x 64 block of mask bits is empty.
     // (A ring of three stages, copies two tiles ahead, measured the same to 2 % slower on every
     // workload and costs 18 KB more LDS.)
-    // Every tile is copied: exchanging per-tile "is any of the 128 rows live" flags between the
-    // waves (tried: through LDS two tiles ahead, and as a bit map built up front from the mask
-    // rows) cost more than the copies it saved, on block-structured masks too.
-    auto iteration = [&](const int t, auto slot_c) __attribute__((always_inline)) {
+    int visits = 0;
+    auto visit = [&](const int t, const int t_next, auto slot_c) __attribute__((always_inline)) {
         constexpr int SLOT = decltype(slot_c)::value;
         constexpr int SLOT2 = SLOT ^ 1;       // the stage freed by the barrier below
         if (even_progress) {
             // The hardware serves the oldest wave first, so of three co-resident work-groups one
             // finishes early and the last runs alone, at a worse rate than three together.  When
             // no other work-group waits for the slot, a wave therefore yields as it advances.
-            if (t == T / 4) __builtin_amdgcn_s_setprio(2);
-            else if (t == T / 2) __builtin_amdgcn_s_setprio(1);
-            else if (t == (3 * T) / 4) __builtin_amdgcn_s_setprio(0);
+            if (visits == n_visits / 4) __builtin_amdgcn_s_setprio(2);
+            else if (visits == n_visits / 2) __builtin_amdgcn_s_setprio(1);
+            else if (visits == (3 * n_visits) / 4) __builtin_amdgcn_s_setprio(0);
         }
+        ++visits;
         wait_vmcnt<0>();          // the copies of tile t (the only ones in flight) have landed
         if (ragged && t == T - 1) zero_tail_rows(t, SLOT);
-        __syncthreads();          // tile t landed for every wave; the stage of tile t - 1 is free
+        __syncthreads();          // tile t landed for every wave; the stage of the previous visit is free
         const u32x2 w2 = mask_words(t, SLOT);
-        if (t + 1 < T) {
-            issue_mask(t + 1, integral_constant<int, SLOT2>{});
-            issue_kv(t + 1, integral_constant<int, SLOT2>{});
+        if (t_next < T) {
+            issue_mask(t_next, integral_constant<int, SLOT2>{});
+            issue_kv(t_next, integral_constant<int, SLOT2>{});
         }
         compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
     };
-    for (int t = 0; t < T; t += 2) {
-        iteration(t, integral_constant<int, 0>{});
-        if (t + 1 < T) iteration(t + 1, integral_constant<int, 1>{});
+    for (int t = t_first; t < T;) {
+        const int tn = next_tile();
+        visit(t, tn, integral_constant<int, 0>{});
+        if (tn >= T) break;
+        t = next_tile();
+        visit(tn, t, integral_constant<int, 1>{});
     }
     wait_vmcnt<0>();              // no copy may outlive the work-group's LDS allocation
 
@@ -534,7 +590,7 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     {
         const int row0 = qt * BM + wave * 32;
         uint16_t *ob = slab(a.out, bi, hi) + (size_t)row0 * o_sn;
-        const uint32_t ebase = lds0 + (uint32_t)(T % NSTAGE) * STAGE_BYTES + wave * 4096;
+        const uint32_t ebase = lds0 + (uint32_t)(visits & 1) * STAGE_BYTES + wave * 4096;
         if constexpr (HDIM == 32) {
             store_block<BF16, 32>(oacc[0], oacc[0], inv, ebase, ob, (int)o_sn, row0, N, lane);
         } else {

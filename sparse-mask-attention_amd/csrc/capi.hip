@@ -77,6 +77,33 @@ const char *sma_strerror(int code)
     }
 }
 
+long long sma_tile_map_words(int N)
+{
+    if (N <= 0) return 0;
+    const long long blocks = (N + 63) / 64, tw = (blocks + 31) / 32;
+    return blocks * 2 * tw;
+}
+
+int sma_tile_map(const uint32_t *mask_packed, uint32_t *tile_map, int B, int H, int N, void *stream)
+{
+    if (B < 0 || H < 0 || N < 0) return SMA_ERR_BAD_SHAPE;
+    const long long slabs = (long long)B * H;
+    if (slabs == 0 || N == 0) return SMA_OK;
+    if (mask_packed == nullptr || tile_map == nullptr) return SMA_ERR_NULL_POINTER;
+    if (misaligned(mask_packed, 4) || misaligned(tile_map, 4)) return SMA_ERR_ALIGNMENT;
+    if (slabs * ((N + 63) / 64) >= (1ll << 31) || N > 131072) return SMA_ERR_BAD_SHAPE;
+    const hipError_t e = sma::launch_tile_map(mask_packed, tile_map, slabs, N, static_cast<hipStream_t>(stream));
+    return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
+}
+
+int sma_pack_mask_map(const uint8_t *mask, uint32_t *packed, uint32_t *tile_map, int B, int H, int N,
+                      void *stream)
+{
+    const int st = sma_pack_mask(mask, packed, B, H, N, stream);
+    if (st != SMA_OK || tile_map == nullptr) return st;
+    return sma_tile_map(packed, tile_map, B, H, N, stream);
+}
+
 int sma_pack_mask(const uint8_t *mask, uint32_t *packed, int B, int H, int N, void *stream)
 {
     if (B < 0 || H < 0 || N < 0) return SMA_ERR_BAD_SHAPE;
@@ -159,10 +186,10 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
     return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
 }
 
-int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_tensor *v,
-                         const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
-                         const sma_tensor *out, float *lse, int B, int H, int N, int D, float scale,
-                         int dtype, void *stream)
+int sma_attn_fwd_map_strided(const sma_tensor *q, const sma_tensor *k, const sma_tensor *v,
+                             const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                             const uint32_t *tile_map, const sma_tensor *out, float *lse, int B, int H,
+                             int N, int D, float scale, int dtype, void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
     if (D != 32 && D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
@@ -175,7 +202,8 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
     // a lane's byte offset into the packed mask of one (b,h) is a 32-bit register
     if ((long long)N * ((N + 31) / 32) * 4 >= (1ll << 32)) return SMA_ERR_BAD_SHAPE;
-    if (misaligned(mask_packed, 4) || (lse && misaligned(lse, 4))) return SMA_ERR_ALIGNMENT;
+    if (misaligned(mask_packed, 4) || (lse && misaligned(lse, 4)) || (tile_map && misaligned(tile_map, 4)))
+        return SMA_ERR_ALIGNMENT;
     if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 
     sma::AttnArgs a;
@@ -193,12 +221,36 @@ int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_ten
     a.D = D;
     a.byte_mask = 0;
     a.mask_out = nullptr;
+    // the map is contiguous [Bm, Hm, ...] with the mask's own Bm, Hm (1 where the mask is shared)
+    a.tile_map = tile_map;
+    const long long map_words = sma_tile_map_words(N);
+    a.map_sh = (H > 1 && mask_stride_h != 0) ? map_words : 0;
+    a.map_sb = (B > 1 && mask_stride_b != 0) ? ((H > 1 && mask_stride_h != 0) ? (long long)H : 1ll) * map_words : 0;
     a.qtiles = (int)qtiles;
     split_scale(scale, &a.q_scale, &a.post_mul);
     last_tile_masks(N, &a.last_mask0, &a.last_mask1);
 
     const hipError_t e = sma::launch_attn_fwd(a, dtype == SMA_DTYPE_BF16, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
+}
+
+int sma_attn_fwd_strided(const sma_tensor *q, const sma_tensor *k, const sma_tensor *v,
+                         const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                         const sma_tensor *out, float *lse, int B, int H, int N, int D, float scale,
+                         int dtype, void *stream)
+{
+    return sma_attn_fwd_map_strided(q, k, v, mask_packed, mask_stride_b, mask_stride_h, nullptr, out, lse, B, H, N,
+                                    D, scale, dtype, stream);
+}
+
+int sma_attn_fwd_map(const void *q, const void *k, const void *v, const uint32_t *mask_packed,
+                     const uint32_t *tile_map, void *out, float *lse, int B, int H, int N, int D,
+                     float scale, int dtype, void *stream)
+{
+    const sma_tensor t[4] = {dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D), dense(out, H, N, D)};
+    const int64_t msh = (int64_t)N * ((N + 31) / 32);
+    return sma_attn_fwd_map_strided(&t[0], &t[1], &t[2], mask_packed, msh * H, msh, tile_map, &t[3], lse, B, H, N, D,
+                                    scale, dtype, stream);
 }
 
 int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const uint8_t *mask,
@@ -237,6 +289,8 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
     a.D = D;
     a.byte_mask = 1;
     a.mask_out = packed_out;
+    a.tile_map = nullptr;
+    a.map_sb = a.map_sh = 0;
     a.qtiles = (int)qtiles;
     split_scale(scale, &a.q_scale, &a.post_mul);
     last_tile_masks(N, &a.last_mask0, &a.last_mask1);

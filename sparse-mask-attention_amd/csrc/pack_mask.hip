@@ -181,7 +181,59 @@ __global__ __launch_bounds__(PACK_THREADS) void pack_short_rows_kernel(const uin
     packed[row] = acc;
 }
 
+// Tile map of a packed mask: for every (slab, block of 64 query rows) one bit per 64-key tile that
+// says "some mask bit of this 64 x 64 block is set" (word group 0) and one that says "every bit of
+// the block is set" (word group 1; only rows and columns below N count).  Layout
+// [slab][row block][2][tw], tw = ceil(T / 32) words, T = ceil(N / 64); bits of tiles >= T are zero.
+// One work-group per (slab, row block): it streams the block's 64 x nw words (coalesced), every
+// thread ORs what its words say into per-key-tile flags in LDS, and the first tw threads write the
+// words.  No atomics on global memory, nothing to clear beforehand, deterministic.
+constexpr int MAP_MAX_TW = 64;      // key tiles per query tile <= 2048, i.e. N <= 131072
+__global__ __launch_bounds__(PACK_THREADS) void tile_map_kernel(const uint32_t *__restrict__ packed,
+                                                                uint32_t *__restrict__ map,
+                                                                int N, int nw, int qblocks, int tw)
+{
+    __shared__ uint32_t some[MAP_MAX_TW], hole[MAP_MAX_TW];       // hole: a valid bit of the tile is clear
+    const int slab = blockIdx.x / qblocks, qt = blockIdx.x - slab * qblocks;
+    if ((int)threadIdx.x < tw) { some[threadIdx.x] = 0u; hole[threadIdx.x] = 0u; }
+    __syncthreads();
+    const int row0 = qt * 64;
+    const int rows = N - row0 < 64 ? N - row0 : 64;
+    const uint32_t *src = packed + ((size_t)slab * N + row0) * nw;
+    const int words = rows * nw;
+    const uint32_t tail = (N & 31) ? ((1u << (N & 31)) - 1u) : 0xffffffffu;     // valid bits of a row's last word
+    for (int i = threadIdx.x; i < words; i += PACK_THREADS) {
+        const int w = i % nw;
+        const uint32_t valid = w == nw - 1 ? tail : 0xffffffffu;
+        const uint32_t x = src[i] & valid;
+        const int kt = w >> 1;
+        const uint32_t bit = 1u << (kt & 31);
+        // most blocks are mixed: look before the (serialising) LDS atomic
+        if (x != 0u && (some[kt >> 5] & bit) == 0u) atomicOr(&some[kt >> 5], bit);
+        if (x != valid && (hole[kt >> 5] & bit) == 0u) atomicOr(&hole[kt >> 5], bit);
+    }
+    __syncthreads();
+    if ((int)threadIdx.x < tw) {
+        const int T = (N + 63) / 64;
+        const int w = threadIdx.x;
+        const uint32_t in_range = (w == tw - 1 && (T & 31)) ? ((1u << (T & 31)) - 1u) : 0xffffffffu;
+        uint32_t *dst = map + ((size_t)slab * qblocks + qt) * 2 * tw;
+        dst[w] = some[w] & in_range;
+        dst[tw + w] = ~hole[w] & in_range;
+    }
+}
+
 }  // namespace
+
+hipError_t launch_tile_map(const uint32_t *packed, uint32_t *map, long long slabs, int N, hipStream_t stream)
+{
+    if (slabs == 0 || N == 0) return hipSuccess;
+    const int nw = (N + 31) / 32, qblocks = (N + 63) / 64, tw = (qblocks + 31) / 32;
+    if (tw > MAP_MAX_TW) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(tile_map_kernel, dim3((unsigned)(slabs * qblocks)), dim3(PACK_THREADS), 0, stream, packed, map,
+                       N, nw, qblocks, tw);
+    return hipGetLastError();
+}
 
 hipError_t launch_pack_mask(const uint8_t *mask, uint32_t *packed, long long rows, int N,
                             hipStream_t stream)

@@ -53,6 +53,11 @@ struct AttnArgs {
     int D;                          // head dim: 32, 64 or 128
     int byte_mask;                  // the mask is the caller's boolean tensor, not packed words
     uint32_t *mask_out;             // byte_mask only: nullptr, or where to leave the packed words [Bm, Hm, N, nw]
+    // packed mask only: nullptr, or the tile map [Bm, Hm, T, 2, ceil(T/32)] (T = ceil(N/64)): per block
+    // of 64 query rows one bit per 64-key tile "some mask bit set", then one bit per key tile "all
+    // mask bits set"; strides between batch entries / heads in words, 0 = shared
+    const uint32_t *tile_map;
+    long long map_sb, map_sh;
     int qtiles;                     // ceil(N / 128): query tiles (work-groups) per (b,h)
     FastDiv div_qtiles, div_H;      // filled in by the launcher
     // exp(scale * s) is evaluated as exp2(post_mul * (q_scale * q) . k): q is multiplied by
@@ -87,5 +92,7 @@ hipError_t launch_attn_fwd(const AttnArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_attn_bwd(const AttnBwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_pack_mask(const uint8_t *mask, uint32_t *packed, long long rows, int N,
                             hipStream_t stream);
+// tile map [slabs, ceil(N/64), 2, ceil(ceil(N/64)/32)] of packed words [slabs, N, ceil(N/32)]
+hipError_t launch_tile_map(const uint32_t *packed, uint32_t *map, long long slabs, int N, hipStream_t stream);
 
 }  // namespace sma

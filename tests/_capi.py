@@ -52,6 +52,14 @@ def load():
         lib.sma_attn_fwd.argtypes = [vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_bwd.restype = ci
         lib.sma_attn_bwd.argtypes = [vp] * 11 + [ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_tile_map_words.restype = ctypes.c_longlong
+        lib.sma_tile_map_words.argtypes = [ci]
+        lib.sma_tile_map.restype = ci
+        lib.sma_tile_map.argtypes = [vp, vp, ci, ci, ci, vp]
+        lib.sma_pack_mask_map.restype = ci
+        lib.sma_pack_mask_map.argtypes = [vp, vp, vp, ci, ci, ci, vp]
+        lib.sma_attn_fwd_map.restype = ci
+        lib.sma_attn_fwd_map.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_bwd_static_ws.restype = ci
         lib.sma_attn_bwd_static_ws.argtypes = [vp] * 10 + [ci, ci, ci, ci, cf, ci, vp]
         tp, i64 = ctypes.POINTER(SmaTensor), ctypes.c_int64
@@ -59,6 +67,8 @@ def load():
         lib.sma_attn_fwd_strided.argtypes = [tp, tp, tp, vp, i64, i64, tp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_bwd_strided.restype = ci
         lib.sma_attn_bwd_strided.argtypes = [tp] * 5 + [vp, vp, i64, i64, tp, tp, tp, vp, ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_attn_fwd_map_strided.restype = ci
+        lib.sma_attn_fwd_map_strided.argtypes = [tp, tp, tp, vp, i64, i64, vp, tp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_fwd_bool_mask.restype = ci
         lib.sma_attn_fwd_bool_mask.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         _lib = lib
@@ -79,6 +89,71 @@ def pack_mask(mask: torch.Tensor) -> torch.Tensor:
     st = lib.sma_pack_mask(mask.data_ptr(), packed.data_ptr(), B, H, N, _stream())
     assert st == SMA_OK, lib.sma_strerror(st)
     return packed
+
+
+def _new_map(Bm, Hm, N, device):
+    """Poisoned tile map tensor [Bm,Hm,T,2,TW] (int32 holding uint32 words)."""
+    lib = load()
+    QT = (N + 63) // 64
+    TW = (QT + 31) // 32
+    assert lib.sma_tile_map_words(N) == QT * 2 * TW
+    return torch.full((Bm, Hm, QT, 2, TW), -1431655766, dtype=torch.int32, device=device)
+
+
+def tile_map(packed: torch.Tensor) -> torch.Tensor:
+    """int32 [B,H,N,nw] packed words -> tile map through sma_tile_map."""
+    lib = load()
+    B, H, N, _ = packed.shape
+    tm = _new_map(B, H, N, packed.device)
+    st = lib.sma_tile_map(packed.data_ptr(), tm.data_ptr(), B, H, N, _stream())
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return tm
+
+
+def pack_mask_map(mask: torch.Tensor):
+    """bool [B,H,N,N] -> (packed, tile map) through sma_pack_mask_map."""
+    lib = load()
+    B, H, N, _ = mask.shape
+    mask = mask.contiguous()
+    packed = torch.full((B, H, N, (N + 31) // 32), -1431655766, dtype=torch.int32, device=mask.device)
+    tm = _new_map(B, H, N, mask.device)
+    st = lib.sma_pack_mask_map(mask.data_ptr(), packed.data_ptr(), tm.data_ptr(), B, H, N, _stream())
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return packed, tm
+
+
+def attn_fwd_map(q, k, v, packed, tm, scale=None, want_lse=False):
+    """Fused forward through sma_attn_fwd_map (tile map of the same mask); returns out (and lse)."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device) if want_lse else None
+    st = lib.sma_attn_fwd_map(q.data_ptr(), k.data_ptr(), v.data_ptr(), packed.data_ptr(),
+                              tm.data_ptr() if tm is not None else None, out.data_ptr(),
+                              lse.data_ptr() if want_lse else None, B, H, N, D, scale, dt, _stream())
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return (out, lse) if want_lse else out
+
+
+def attn_fwd_map_strided(q, k, v, packed, tm, out=None, scale=None, want_lse=False):
+    """sma_attn_fwd_map_strided: as attn_fwd_strided, with the tile map [Bm,Hm,QT,2,TW] of `packed`."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    if out is None:
+        out = torch.full((B, H, N, D), float("nan"), dtype=q.dtype, device=q.device)
+    lse = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device) if want_lse else None
+    msb, msh = _mask_strides(packed, B, H)
+    tq, tk, tv, to = (SmaTensor.of(t) for t in (q, k, v, out))
+    st = lib.sma_attn_fwd_map_strided(tq, tk, tv, packed.data_ptr(), msb, msh, tm.data_ptr(), to,
+                                      lse.data_ptr() if want_lse else None, B, H, N, D, scale, dt, _stream())
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return (out, lse) if want_lse else out
 
 
 def attn_fwd(q, k, v, packed, scale=None, want_lse=False):

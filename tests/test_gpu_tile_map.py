@@ -1,0 +1,130 @@
+"""GPU parity of the tile map (sma_tile_map, sma_pack_mask_map) against the oracle, bit for bit, and
+of the forward that walks it (sma_attn_fwd_map): the same output and lse, bit for bit, as the forward
+that visits every tile, on masks with empty blocks, empty block rows, full blocks and ragged
+edges, at all head dims and both dtypes, and on the benchmark workloads at full size."""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import _capi
+import harness
+from oracle import sma_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _block_mask(B, H, N, g, keep=0.3, inner=1.0, bs=64):
+    nb = (N + bs - 1) // bs
+    blocks = torch.rand(B, H, nb, nb, generator=g) < keep
+    m = blocks.repeat_interleave(bs, 2).repeat_interleave(bs, 3)[:, :, :N, :N].contiguous()
+    if inner < 1.0:
+        m &= torch.rand(B, H, N, N, generator=g) < inner
+    return m
+
+
+def _masks(N, g):
+    yield "random 2 %", torch.rand(2, 2, N, N, generator=g) < 0.02
+    yield "blocks of 64, some full", _block_mask(2, 2, N, g)
+    yield "blocks of 64, thinned", _block_mask(2, 2, N, g, inner=0.5)
+    yield "blocks of 32", _block_mask(2, 2, N, g, keep=0.15, bs=32)
+    yield "causal", torch.tril(torch.ones(N, N, dtype=torch.bool)).expand(2, 2, N, N).contiguous()
+    yield "all true", torch.ones(1, 2, N, N, dtype=torch.bool)
+    yield "all false", torch.zeros(1, 2, N, N, dtype=torch.bool)
+    band = (torch.arange(N)[:, None] - torch.arange(N)[None, :]).abs() < 40
+    yield "band", band.expand(1, 2, N, N).contiguous()
+    late = torch.zeros(1, 2, N, N, dtype=torch.bool)
+    late[..., N - 1] = True                                       # only the last key: one live tile at the end
+    yield "last key only", late
+
+
+@pytest.mark.parametrize("N", [1, 17, 64, 65, 128, 129, 200, 256, 333, 512, 1000])
+def test_tile_map_matches_the_oracle(dev, N):
+    g = torch.Generator().manual_seed(N)
+    for name, mask in _masks(N, g):
+        packed, tm = _capi.pack_mask_map(mask.to(dev))
+        torch.cuda.synchronize()
+        want = O.tile_map_ref(mask).view(np.int32)
+        assert np.array_equal(packed.cpu().numpy(), O.pack_mask_ref(mask)), (name, N)
+        assert np.array_equal(tm.cpu().numpy(), want), (name, N)
+        # the same from words that carry dirt in their pad bits
+        if N % 32:
+            dirty = packed.clone()
+            dirty[..., -1] |= -(1 << (N % 32))
+            assert np.array_equal(_capi.tile_map(dirty).cpu().numpy(), want), (name, N, "dirty pad bits")
+
+
+def test_tile_map_with_more_than_32_key_tiles(dev):
+    N = 64 * 33 + 5
+    g = torch.Generator().manual_seed(1)
+    mask = torch.rand(1, 1, N, N, generator=g) < 0.0005
+    mask[0, 0, :64, 64 * 32: 64 * 33] = True
+    packed, tm = _capi.pack_mask_map(mask.to(dev))
+    torch.cuda.synchronize()
+    assert np.array_equal(tm.cpu().numpy(), O.tile_map_ref(mask).view(np.int32))
+    q, k, v = (torch.randn(1, 1, N, 64, generator=g).half().to(dev) for _ in range(3))
+    a, la = _capi.attn_fwd(q, k, v, packed, want_lse=True)
+    b, lb = _capi.attn_fwd_map(q, k, v, packed, tm, want_lse=True)
+    torch.cuda.synchronize()
+    assert torch.equal(a, b) and torch.equal(la, lb)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("N", [64, 200, 333, 512])
+def test_forward_with_map_equals_forward_without(dev, N, D, dtype):
+    g = torch.Generator().manual_seed(1000 * D + N)
+    q, k, v = (torch.randn(2, 2, N, D, generator=g).to(dtype).to(dev) for _ in range(3))
+    for name, mask in _masks(N, g):
+        B, H = mask.shape[:2]
+        packed, tm = _capi.pack_mask_map(mask.to(dev))
+        qq, kk, vv = q[:B], k[:B], v[:B]
+        want, want_lse = _capi.attn_fwd(qq, kk, vv, packed, want_lse=True)
+        got, lse = _capi.attn_fwd_map(qq, kk, vv, packed, tm, want_lse=True)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want) and torch.equal(lse, want_lse), (name, N, D, dtype)
+        ref = O.sparse_attention_ref(qq.float().cpu(), kk.float().cpu(), vv.float().cpu(), mask)
+        rtol = 1e-2 if dtype == torch.float16 else 2e-2
+        assert torch.allclose(got.float().cpu(), ref, atol=1e-2, rtol=rtol), (name, N, D, dtype)
+
+
+def test_shared_mask_and_strided_tensors(dev):
+    g = torch.Generator().manual_seed(3)
+    B, H, N = 3, 4, 300
+    buf = torch.randn(B, N, 3, H, 64, generator=g).half().to(dev)
+    q, k, v = (buf[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    for shape in [(1, 1), (B, 1), (1, H)]:
+        mask = _block_mask(shape[0], shape[1], N, g, keep=0.3, inner=0.6)
+        packed, tm = _capi.pack_mask_map(mask.to(dev))
+        want = _capi.attn_fwd_strided(q, k, v, packed)
+        got = _capi.attn_fwd_map_strided(q, k, v, packed, tm)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want), shape
+        ref = O.sparse_attention_ref(q.float().cpu(), k.float().cpu(), v.float().cpu(), mask.expand(B, H, N, N))
+        assert torch.allclose(got.float().cpu(), ref, atol=1e-2, rtol=1e-2), shape
+
+
+@pytest.mark.parametrize("name", ["C2", "C3", "C4", "C5"])
+def test_benchmark_workloads_with_map(dev, name):
+    w = harness.WORKLOADS[name]
+    q, k, v, mask = harness.make_inputs(w, seed=42)
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    packed, tm = _capi.pack_mask_map(md)
+    want, want_lse = _capi.attn_fwd(qd, kd, vd, packed, want_lse=True)
+    got, lse = _capi.attn_fwd_map(qd, kd, vd, packed, tm, want_lse=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and torch.equal(lse, want_lse)
+    # the map itself, on the GPU: blocks with a set bit, blocks without a hole
+    QT = T = (w.N + 63) // 64
+    pad = torch.zeros(w.B, w.H, QT * 64, T * 64, dtype=torch.bool, device=dev)
+    pad[:, :, :w.N, :w.N] = md
+    some = pad.view(w.B, w.H, QT, 64, T, 64).any(dim=5).any(dim=3)
+    pad.fill_(True)
+    pad[:, :, :w.N, :w.N] = md
+    full = pad.view(w.B, w.H, QT, 64, T, 64).all(dim=5).all(dim=3)
+    bits = torch.arange(T, device=dev)
+    words = tm.view(w.B, w.H, QT, 2, -1).long() & 0xFFFFFFFF
+    got_some = ((words[:, :, :, 0, :].repeat_interleave(32, -1)[..., :T] >> (bits % 32)) & 1).bool()
+    got_full = ((words[:, :, :, 1, :].repeat_interleave(32, -1)[..., :T] >> (bits % 32)) & 1).bool()
+    assert torch.equal(got_some, some) and torch.equal(got_full, full)

@@ -239,3 +239,63 @@ def test_backward_all_true_mask_equals_dense_sdpa_autograd():
     dq, dk, dv = O.sparse_attention_bwd_ref(q, k, v, mask, do)
     for got, ref in ((dq, qa.grad), (dk, ka.grad), (dv, va.grad)):
         assert torch.allclose(got, ref, atol=1e-10, rtol=1e-8)
+
+
+# ---------------------------------------------------------------------------
+# tile map
+# ---------------------------------------------------------------------------
+
+@pytest.mark.parametrize("N", [1, 63, 64, 65, 127, 128, 129, 200, 333])
+def test_tile_map_equals_literal_loops(N):
+    g = torch.Generator().manual_seed(N)
+    mask = torch.rand(1, 2, N, N, generator=g) < 0.02            # sparse enough for empty blocks
+    mask[0, 0, : min(N, 64), : min(N, 64)] = True                # and one full block
+    assert np.array_equal(O.tile_map_ref(mask), O.tile_map_loops(mask))
+
+
+def test_tile_map_known_answers():
+    N = 200                                                      # 4 row blocks, 4 key tiles (last: 8 wide)
+    assert O.tile_map_shape(N) == (4, 2, 1)
+    ones = O.tile_map_ref(torch.ones(1, 1, N, N, dtype=torch.bool))
+    assert (ones == 0xF).all()                                   # four tiles live and full, the ragged ones too
+    zeros = O.tile_map_ref(torch.zeros(1, 1, N, N, dtype=torch.bool))
+    assert (zeros == 0).all()
+    one = torch.zeros(1, 1, N, N, dtype=torch.bool)
+    one[0, 0, 130, 70] = True                                    # row block 2, key tile 1
+    m = O.tile_map_ref(one)
+    assert m[0, 0, 2, 0, 0] == 2 and m.sum() == 2                # one live bit, nothing full
+    hole = torch.ones(1, 1, N, N, dtype=torch.bool)
+    hole[0, 0, 5, 199] = False                                   # row block 0, key tile 3
+    m = O.tile_map_ref(hole)
+    assert m[0, 0, 0, 0, 0] == 0xF and m[0, 0, 0, 1, 0] == 0x7 and m[0, 0, 1, 1, 0] == 0xF
+    # more than 32 key tiles: a second word
+    N = 64 * 33
+    assert O.tile_map_shape(N) == (33, 2, 2)
+    last = torch.zeros(1, 1, N, N, dtype=torch.bool)
+    last[0, 0, 0, N - 1] = True
+    m = O.tile_map_ref(last)
+    assert m[0, 0, 0, 0, 1] == 1 and m[0, 0, 0, 0, 0] == 0 and m.sum() == 1
+
+
+def test_tiles_called_empty_do_not_matter():
+    """Clearing what the map calls empty changes nothing, and every block it calls full is all True."""
+    g = torch.Generator().manual_seed(5)
+    N = 300
+    blocks = torch.rand(1, 2, 5, 5, generator=g) < 0.4
+    mask = blocks.repeat_interleave(64, 2).repeat_interleave(64, 3)[:, :, :N, :N] & (torch.rand(1, 2, N, N, generator=g) < 0.7)
+    mask[0, 1, 128:192, 64:128] = True
+    m = O.tile_map_ref(mask)
+    QT, _, TW = O.tile_map_shape(N)
+    kept = torch.zeros_like(mask)
+    for h in range(2):
+        for qt in range(QT):
+            for t in range((N + 63) // 64):
+                live = (int(m[0, h, qt, 0, t // 32]) >> (t % 32)) & 1
+                full = (int(m[0, h, qt, 1, t // 32]) >> (t % 32)) & 1
+                blk = mask[0, h, 64 * qt:64 * qt + 64, 64 * t:64 * t + 64]
+                if live:
+                    kept[0, h, 64 * qt:64 * qt + 64, 64 * t:64 * t + 64] = blk
+                if full:
+                    assert blk.all() and live
+    assert torch.equal(kept, mask)
+    assert (int(m[0, 1, 2, 1, 0]) >> 1) & 1
