@@ -190,10 +190,9 @@ int sma_attn_fwd_map_strided(const sma_tensor *q, const sma_tensor *k, const sma
  *
  *   q, k, v, out    contiguous [B,H,N,D], D = 32, 64 or 128; 16 <= N <= 46340
  *   mask            uint8 [Bm,Hm,N,N] with Bm in {1,B}, Hm in {1,H}, rows contiguous, at any byte
- *                   address; every byte must be 0 or 1 (torch.bool storage; unlike sma_pack_mask,
- *                   other non-zero values are not accepted); mask_stride_b / mask_stride_h in
- *                   BYTES, 0 = shared between batch entries / heads.  No byte outside the mask is
- *                   read.
+ *                   address; a byte counts as "attend" when it is non-zero, as in sma_pack_mask;
+ *                   mask_stride_b / mask_stride_h in BYTES, 0 = shared between batch entries /
+ *                   heads.  No byte outside the mask is read.
  *   lse             NULL or float [B,H,N]
  *   packed_out      NULL, or uint32 [Bm,Hm,N,ceil(N/32)] (contiguous): receives exactly what
  *                   sma_pack_mask would write for this mask, as a by-product, for callers who

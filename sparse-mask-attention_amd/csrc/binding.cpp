@@ -4,8 +4,11 @@
 // (csrc/binding.cpp:9-18 `forward`, csrc/binding.cpp:49 `pack_mask`, registered at
 // csrc/binding.cpp:68-71) so that python/sparse_attention.py can stay as it is:
 //
-//   forward(q, k, v, mask_packed, out, lse, scale, is_training) -> None
+//   forward(q, k, v, mask_packed, out, lse, scale, is_training, tile_map=None) -> None
 //   pack_mask(mask) -> int32 Tensor [B, H, N, ceil(N/32)]
+//   tile_map(mask_packed) -> int32 Tensor [B, H, ceil(N/64), 2, ceil(ceil(N/64)/32)]   (not in the
+//       reference: which 64 x 64 blocks of the mask hold a set bit / nothing but set bits; passed to
+//       `forward` as tile_map, key tiles without a set bit are neither loaded nor computed)
 //   backward(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, scale) -> None   (called by the
 //       reference's Python API, python/sparse_attention.py:91-94, but absent from its binding)
 //   forward_bool_mask(q, k, v, mask, out, lse, scale, is_training, packed_out=None) -> None   (not in
@@ -69,7 +72,8 @@ void mask_strides(const torch::Tensor &mp, const torch::Tensor &q, int64_t *sb, 
 
 void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,
              const torch::Tensor &mask_packed, torch::Tensor out,
-             const c10::optional<torch::Tensor> &lse, double scale, bool is_training)
+             const c10::optional<torch::Tensor> &lse, double scale, bool is_training,
+             const c10::optional<torch::Tensor> &tile_map)
 {
     TORCH_CHECK(q.is_cuda(), "q must be a GPU tensor");
     TORCH_CHECK(q.dim() == 4, "q must be 4D [B, H, N, D]");
@@ -95,14 +99,25 @@ void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor
         lse_ptr = lse->data_ptr<float>();
     }
     TORCH_CHECK(B <= INT32_MAX && H <= INT32_MAX && N <= INT32_MAX, "extent too large");
+    const uint32_t *map_ptr = nullptr;
+    if (tile_map.has_value() && tile_map->defined()) {
+        const torch::Tensor &m = *tile_map;
+        const int64_t T = (N + 63) / 64;
+        TORCH_CHECK(m.device() == q.device() && m.scalar_type() == at::kInt && m.dim() == 5 &&
+                        m.size(0) == mask_packed.size(0) && m.size(1) == mask_packed.size(1) && m.size(2) == T &&
+                        m.size(3) == 2 && m.size(4) == (T + 31) / 32 && m.is_contiguous(),
+                    "tile_map must be the contiguous int32 result of tile_map(mask_packed)");
+        map_ptr = reinterpret_cast<const uint32_t *>(m.data_ptr<int32_t>());
+    }
 
     const c10::DeviceGuard guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
-    const int st = sma_attn_fwd_strided(&tq, &tk, &tv,
-                                        reinterpret_cast<const uint32_t *>(mask_packed.data_ptr<int32_t>()),
-                                        msb, msh, &to, lse_ptr, (int)B, (int)H, (int)N, (int)D, (float)scale,
-                                        dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
-    check_status(st, "sma_attn_fwd_strided");
+    const int st = sma_attn_fwd_map_strided(&tq, &tk, &tv,
+                                            reinterpret_cast<const uint32_t *>(mask_packed.data_ptr<int32_t>()),
+                                            msb, msh, map_ptr, &to, lse_ptr, (int)B, (int)H, (int)N, (int)D,
+                                            (float)scale, dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16,
+                                            stream);
+    check_status(st, "sma_attn_fwd_map_strided");
 }
 
 // Limits of sma_attn_fwd_bool_mask, so that callers can choose between it and pack_mask + forward
@@ -234,6 +249,25 @@ torch::Tensor pack_mask(const torch::Tensor &mask)
     return packed;
 }
 
+// tile_map(mask_packed): [Bm, Hm, N, ceil(N/32)] int32 -> [Bm, Hm, T, 2, ceil(T/32)] int32, T = ceil(N/64).
+torch::Tensor tile_map(const torch::Tensor &mask_packed)
+{
+    TORCH_CHECK(mask_packed.is_cuda(), "mask_packed must be a GPU tensor");
+    TORCH_CHECK(mask_packed.scalar_type() == at::kInt && mask_packed.dim() == 4 && mask_packed.is_contiguous(),
+                "mask_packed must be a contiguous int32 [B, H, N, ceil(N/32)] tensor");
+    const int64_t B = mask_packed.size(0), H = mask_packed.size(1), N = mask_packed.size(2);
+    TORCH_CHECK(mask_packed.size(3) == (N + 31) / 32, "mask_packed must be [B, H, N, ceil(N/32)]");
+    TORCH_CHECK(B <= INT32_MAX && H <= INT32_MAX && N <= 131072, "extent too large");
+    const int64_t T = (N + 63) / 64;
+    const c10::DeviceGuard guard(mask_packed.device());
+    torch::Tensor map = torch::empty({B, H, T, 2, (T + 31) / 32}, mask_packed.options());    // every word is written
+    hipStream_t stream = c10::hip::getCurrentHIPStream(mask_packed.device().index()).stream();
+    const int st = sma_tile_map(reinterpret_cast<const uint32_t *>(mask_packed.data_ptr<int32_t>()),
+                                reinterpret_cast<uint32_t *>(map.data_ptr<int32_t>()), (int)B, (int)H, (int)N, stream);
+    check_status(st, "sma_tile_map");
+    return map;
+}
+
 }  // namespace
 
 PYBIND11_MODULE(sparse_attn_cuda, m)
@@ -241,7 +275,10 @@ PYBIND11_MODULE(sparse_attn_cuda, m)
     m.doc() = "sparse-mask attention for MI355X (gfx950): pybind shim over libsma_hip.so";
     m.def("forward", &forward, "Sparse-mask attention forward", py::arg("q"), py::arg("k"),
           py::arg("v"), py::arg("mask_packed"), py::arg("out"), py::arg("lse"), py::arg("scale"),
-          py::arg("is_training"));
+          py::arg("is_training"), py::arg("tile_map") = py::none());
+    m.def("tile_map", &tile_map,
+          "Which 64 x 64 blocks of a packed mask hold a set bit / only set bits (pass to forward as tile_map)",
+          py::arg("mask_packed"));
     m.def("backward", &backward, "Sparse-mask attention backward (dq, dk, dv are overwritten)",
           py::arg("dout"), py::arg("q"), py::arg("k"), py::arg("v"), py::arg("out"), py::arg("lse"),
           py::arg("mask_packed"), py::arg("dq"), py::arg("dk"), py::arg("dv"), py::arg("scale"));

@@ -36,7 +36,13 @@ What differs from the reference, on purpose:
   N >= 16) one launch reads the bool mask itself and forms the packed words tile by
   tile, which is 15-35 % faster than pack + attention; under autograd the same launch also leaves
   the packed words behind for the backward.  Otherwise the mask is packed as the reference does.
-  Results are bit-identical either way.
+  Results are bit-identical either way; both ways count any non-zero mask byte as True, so a bool
+  tensor made by ``view`` from bytes other than 0 and 1 is read the same by both.
+* Block-structured masks (sliding window, block-sparse, causal): ``tile_map(mask_packed)`` says
+  which 64 x 64 blocks of the mask hold a set bit; given as ``tile_map=`` together with
+  ``mask_packed=`` the forward neither loads nor computes the key tiles that hold none (the
+  reference skips such a tile only after loading it, ``csrc/sparse_attention.cu:211,238-252``).
+  Worth it for a mask that is used many times; ``tile_map`` returns None when no block is empty.
 * ``.backward()`` works.  The reference calls a ``sparse_attn_cuda.backward`` that was never
   written (:91-94); here that function exists (two HIP kernels, dQ and dK/dV, from the saved
   log-sum-exp and the packed mask).  ``backward_recompute`` states the same gradients with PyTorch
@@ -108,7 +114,7 @@ class SparseAttentionFunction(Function):
     does not apply."""
 
     @staticmethod
-    def forward(ctx, q, k, v, mask_packed, mask_bool, scale, seq_len):
+    def forward(ctx, q, k, v, mask_packed, mask_bool, scale, seq_len, tile_map=None):
         _require_ext(q)
         B, H, N, _ = q.shape
         q, k, v = _rows(q), _rows(k), _rows(v)
@@ -124,7 +130,7 @@ class SparseAttentionFunction(Function):
                 ctx.scale = scale
                 return out
             mask_packed = pack_mask(mask_bool)
-        sparse_attn_cuda.forward(q, k, v, mask_packed, out, lse, scale, True)
+        sparse_attn_cuda.forward(q, k, v, mask_packed, out, lse, scale, True, tile_map)
         ctx.save_for_backward(q, k, v, out, lse, mask_packed)
         ctx.scale = scale
         return out
@@ -136,7 +142,7 @@ class SparseAttentionFunction(Function):
         # the call the reference makes at python/sparse_attention.py:91-94
         sparse_attn_cuda.backward(_rows(dout.to(q.dtype)), q, k, v, out, lse, mask_packed,
                                   dq, dk, dv, ctx.scale)
-        return dq, dk, dv, None, None, None, None
+        return dq, dk, dv, None, None, None, None, None
 
 
 def backward_recompute(q, k, v, out, lse, mask_bool, dout, scale):
@@ -202,7 +208,7 @@ def _pad_head_dim(q, k, v):
     return tuple(torch.nn.functional.pad(t, pad) for t in (q, k, v))
 
 
-def sparse_attention(q, k, v, mask, mask_packed=None):
+def sparse_attention(q, k, v, mask, mask_packed=None, tile_map=None):
     """Masked attention with autograd support.
 
     q, k, v: ``[B, H, N, D]`` (D = 32, 64 or 128; other D <= 128 are zero-padded) bf16 / fp16 / fp32;  mask: bool ``[B, H, N, N]``, True = keep
@@ -211,13 +217,15 @@ def sparse_attention(q, k, v, mask, mask_packed=None):
 
     ``mask_packed`` (optional, not in the reference): the result of ``pack_mask(mask)`` kept from an
     earlier call with the same mask; packing (as much HBM traffic as the attention itself at
-    N = 512) is then skipped and ``mask`` may be None.
+    N = 512) is then skipped and ``mask`` may be None.  ``tile_map`` (optional, with ``mask_packed``):
+    the result of ``tile_map(mask_packed)``; key tiles in which the mask keeps nothing are skipped.
     """
     _check_inputs(q, k, v, mask, mask_packed)
+    assert tile_map is None or mask_packed is not None, "tile_map belongs to a mask_packed"
     _require_ext(q)
     if not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)):
         # nothing will be differentiated: no LSE, and the mask can be read without packing it
-        return sparse_attention_func(q, k, v, mask, mask_packed)
+        return sparse_attention_func(q, k, v, mask, mask_packed, tile_map)
     B, H, N, D = q.shape
     scale = 1.0 / math.sqrt(D)
 
@@ -226,16 +234,17 @@ def sparse_attention(q, k, v, mask, mask_packed=None):
         q, k, v = q.bfloat16(), k.bfloat16(), v.bfloat16()
 
     q, k, v = _pad_head_dim(q, k, v)              # differentiable: the gradients are sliced back
-    out = SparseAttentionFunction.apply(q, k, v, mask_packed, mask, scale, N)[..., :D]
+    out = SparseAttentionFunction.apply(q, k, v, mask_packed, mask, scale, N, tile_map)[..., :D]
 
     if orig_dtype == torch.float32:
         out = out.float()
     return out
 
 
-def sparse_attention_func(q, k, v, mask, mask_packed=None):
+def sparse_attention_func(q, k, v, mask, mask_packed=None, tile_map=None):
     """Inference-only variant of :func:`sparse_attention`: no autograd graph, no LSE."""
     _check_inputs(q, k, v, mask, mask_packed)
+    assert tile_map is None or mask_packed is not None, "tile_map belongs to a mask_packed"
     _require_ext(q)
     D = q.shape[-1]
     scale = 1.0 / math.sqrt(D)
@@ -255,7 +264,7 @@ def sparse_attention_func(q, k, v, mask, mask_packed=None):
                 return (out[..., :D].float() if orig_dtype == torch.float32 else out[..., :D])
             mask_packed = pack_mask(mask)
         out = torch.empty_like(q)
-        sparse_attn_cuda.forward(q, k, v, mask_packed, out, None, scale, False)
+        sparse_attn_cuda.forward(q, k, v, mask_packed, out, None, scale, False, tile_map)
         out = out[..., :D]
 
     if orig_dtype == torch.float32:
@@ -272,6 +281,22 @@ def pack_mask(mask: torch.Tensor) -> torch.Tensor:
     A mask shared between batch entries / heads is passed (and packed) as ``[1 or B, 1 or H, N, N]``."""
     _require_ext(mask)
     return sparse_attn_cuda.pack_mask(mask)
+
+
+def tile_map(mask_packed: torch.Tensor):
+    """Occupancy of the 64 x 64 blocks of a packed mask, for ``sparse_attention(..., mask_packed=,
+    tile_map=)``: int32 ``[B, H, T, 2, ceil(T/32)]`` with T = ceil(N/64); per block of 64 query rows
+    one bit per 64-key tile "some entry kept", then one bit per tile "every entry kept".  Returns
+    None when every block holds a kept entry (nothing could be skipped).  Synchronises with the
+    device once, to look at that; meant to be called once for a mask that is used many times."""
+    _require_ext(mask_packed)
+    tm = sparse_attn_cuda.tile_map(mask_packed)
+    T = tm.shape[2]
+    live = tm[:, :, :, 0, :]
+    every = torch.full((live.shape[-1],), -1, dtype=torch.int32, device=tm.device)
+    if T % 32:
+        every[-1] = (1 << (T % 32)) - 1
+    return None if bool((live == every).all()) else tm
 
 
 def generate_random_sparse_mask(B, H, N, sparsity=0.75, device="cuda"):

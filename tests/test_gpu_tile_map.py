@@ -128,3 +128,33 @@ def test_benchmark_workloads_with_map(dev, name):
     got_some = ((words[:, :, :, 0, :].repeat_interleave(32, -1)[..., :T] >> (bits % 32)) & 1).bool()
     got_full = ((words[:, :, :, 1, :].repeat_interleave(32, -1)[..., :T] >> (bits % 32)) & 1).bool()
     assert torch.equal(got_some, some) and torch.equal(got_full, full)
+
+
+def test_python_api_with_tile_map(dev):
+    """tile_map() through the module: None for a mask without empty blocks; with a map, the forward
+    (inference and autograd) gives bit for bit what it gives without, and gradients still flow."""
+    import importlib
+    sa = importlib.import_module("python.sparse_attention")
+    g = torch.Generator().manual_seed(11)
+    B, H, N = 2, 3, 320
+    q, k, v = (torch.randn(B, H, N, 64, generator=g).half().to(dev) for _ in range(3))
+    dense = (torch.rand(B, H, N, N, generator=g) < 0.3).to(dev)
+    assert sa.tile_map(sa.pack_mask(dense)) is None
+    mask = _block_mask(B, H, N, g, keep=0.3, inner=0.8).to(dev)
+    packed = sa.pack_mask(mask)
+    tm = sa.tile_map(packed)
+    assert tm is not None and tuple(tm.shape) == (B, H, 5, 2, 1) and tm.dtype == torch.int32
+    assert np.array_equal(tm.cpu().numpy(), O.tile_map_ref(mask.cpu()).view(np.int32))
+    want = sa.sparse_attention_func(q, k, v, None, mask_packed=packed)
+    got = sa.sparse_attention_func(q, k, v, None, mask_packed=packed, tile_map=tm)
+    assert torch.equal(got, want)
+    leaves = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    out = sa.sparse_attention(*leaves, None, mask_packed=packed, tile_map=tm)
+    assert torch.equal(out.detach(), want)
+    out.sum().backward()
+    torch.cuda.synchronize()
+    assert all(torch.isfinite(t.grad.float()).all() and t.grad.abs().sum() > 0 for t in leaves)
+    with pytest.raises(AssertionError):
+        sa.sparse_attention_func(q, k, v, mask, tile_map=tm)          # a map without its packed mask
+    with pytest.raises(RuntimeError):
+        sa.sparse_attn_cuda.forward(q, k, v, packed, torch.empty_like(q), None, 0.125, False, tm[:, :, :4])
