@@ -12,13 +12,22 @@ timed as well and reported beside it.  The headline value is dense-equivalent TF
 
 Prints ONE JSON line.  Besides the whole-step figure it carries
   roofline      the dominant kernel of the step alone, from stream-event timing of back-to-back
-                launches on the launch stream: the forward that reads the boolean mask (100.7 MB of
-                compulsory traffic for 12.9 GFLOP on the headline workload, 128 FLOP/B, i.e. on the
-                HBM side of the roofline) or, where that does not apply, the packed-mask forward;
-  roofline_attn the packed-mask forward kernel alone against the dense FP16 MFMA peak;
+                launches on the launch stream: the forward that reads the boolean mask or, where
+                that does not apply, the packed-mask forward.  `frac` is the fraction of the dense
+                FP16/BF16 MFMA peak in dense-equivalent FLOP (the figure the target is written in);
+                the HBM side is in `hbm_*` (100.7 MB of compulsory traffic for 12.9 GFLOP on the
+                headline workload, 128 FLOP/B: below the ridge at 315);
+  roofline_attn the packed-mask forward kernel alone against the MFMA peak (with the tile map of the
+                mask where the mask has empty blocks);
   roofline_pack the packer alone against the HBM peak;
   roofline_bwd  the backward (its two kernels, one call) against the MFMA peak, 2.5 x the forward's FLOP;
   cpu_baseline  the oracle's PyTorch formulation of the same workload on the host cores.
+Every roofline carries two timings.  The plain ones repeat the launch on the same tensors, as the
+reference's protocol does (run.py:172-183): the working set of the headline workload (57 to 101 MB)
+then stays in the 256 MB last-level cache between launches, and the "HBM" fractions computed from it
+are fractions of the HBM peak served partly from that cache.  The `*_cold` ones rotate through
+enough distinct copies of all tensors (more than 512 MB in total) that every launch finds none of
+its data cached: those are HBM figures.
 """
 import argparse
 import ctypes
@@ -52,6 +61,34 @@ def event_time_ms(fn, warmup, repeat, torch):
     end.record()
     torch.cuda.synchronize()
     return start.elapsed_time(end) / repeat
+
+
+def cold_time_ms(make_call, n_sets, warmup, repeat, torch):
+    """Mean ms per call when consecutive calls use different copies of every tensor: make_call(i)
+    returns the call for copy i, n_sets copies exceed the caches, so no call finds its inputs (or
+    the lines of its outputs) resident."""
+    calls = [make_call(i) for i in range(n_sets)]
+    for i in range(max(warmup, n_sets)):
+        calls[i % n_sets]()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    end = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for i in range(repeat):
+        calls[i % n_sets]()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / repeat
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def measured_traffic(workload, *kernels):
@@ -141,9 +178,12 @@ def main():
 
     # ---- the two kernels on their own: back-to-back launches between stream events ----
     packed = ext.pack_mask(md)
+    tmap = sa.tile_map(packed)          # None unless the mask has 64 x 64 blocks without a kept entry
     out = torch.empty_like(qd)
     reps = max(50, args.steps)
-    attn_ms = event_time_ms(lambda: ext.forward(qd, kd, vd, packed, out, None, scale, False), 10, reps, torch)
+    attn_ms = event_time_ms(lambda: ext.forward(qd, kd, vd, packed, out, None, scale, False, tmap), 10, reps, torch)
+    attn_nomap_ms = (event_time_ms(lambda: ext.forward(qd, kd, vd, packed, out, None, scale, False), 10, reps, torch)
+                     if tmap is not None else attn_ms)
     # the packer through the C ABI into a preallocated buffer (no allocator in the loop)
     lib = ctypes.CDLL(os.path.join(PKG, "libsma_hip.so"))
     lib.sma_pack_mask.argtypes = [ctypes.c_void_p, ctypes.c_void_p, ctypes.c_int, ctypes.c_int,
@@ -163,6 +203,23 @@ def main():
     bwd_ms = event_time_ms(lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale),
                            5, reps, torch)
     bwd_tflops = w.bwd_dense_flops / (bwd_ms * 1e-3) / 1e12
+
+    # ---- the same kernels with nothing cached: rotate through copies of every tensor (> 512 MB) ----
+    set_bytes = 4 * qd.numel() * qd.element_size() + md.numel() + packed.numel() * 4
+    n_sets = max(3, -(-(640 << 20) // set_bytes))
+    copies = [(qd.clone(), kd.clone(), vd.clone(), md.clone(), packed.clone(), torch.empty_like(qd))
+              for _ in range(n_sets)]
+    attn_cold_ms = cold_time_ms(lambda i: (lambda c=copies[i]: ext.forward(c[0], c[1], c[2], c[4], c[5], None, scale,
+                                                                            False, tmap)), n_sets, 10, reps, torch)
+    pack_cold_ms = cold_time_ms(lambda i: (lambda c=copies[i]: lib.sma_pack_mask(c[3].data_ptr(), c[4].data_ptr(),
+                                                                                 w.B, w.H, w.N, stream)),
+                                n_sets, 10, reps, torch)
+    fused_cold_ms = None
+    if one_launch:
+        fused_cold_ms = cold_time_ms(lambda i: (lambda c=copies[i]: ext.forward_bool_mask(c[0], c[1], c[2], c[3], c[5],
+                                                                                          None, scale, False)),
+                                     n_sets, 10, reps, torch)
+    del copies
 
     # FLOP the kernel really executes: 32-row x 64-key blocks of the mask that hold a set bit
     # (a wavefront skips the others), 4*32*64*D each, so that skipping is not mistaken for MFMA speed
@@ -185,6 +242,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": (round(value / PUBLISHED_TFLOPS[w.name], 3) if w.name in PUBLISHED_TFLOPS else None),
+        "vs_baseline_note": "the published figure is the reference's kernel on an RTX 3080 (README.md:13): other hardware",
         "dtype": "fp16" if w.dtype == torch.float16 else "bf16",
         "data": "synthetic",
         "config": {"workload": f"{w.name}: B={w.B} H={w.H} N={w.N} D={w.D} {w.mask_kind} mask keep_p={w.keep_prob}",
@@ -195,6 +253,10 @@ def main():
         "step_pack_then_attention_ms": round(two_launch_ms, 5),
         "step_pack_then_attention_tflops": round(w.dense_flops / (two_launch_ms * 1e-3) / 1e12, 3),
         "attn_kernel_ms": round(attn_ms, 5),
+        "attn_kernel_without_tile_map_ms": round(attn_nomap_ms, 5),
+        "attn_kernel_cold_ms": round(attn_cold_ms, 5),
+        "pack_kernel_cold_ms": round(pack_cold_ms, 5),
+        "cold_sets": n_sets,
         "attn_kernel_tflops": round(attn_tflops, 2),
         "attn_kernel_hbm_gbps": round(w.attn_bytes / (attn_ms * 1e-3) / 1e9, 1),
         "attn_kernel_executed_tflops": round(executed_flops / (attn_ms * 1e-3) / 1e12, 2),
@@ -202,13 +264,20 @@ def main():
         "pack_kernel_ms": round(pack_ms, 5),
         "backward_ms": round(bwd_ms, 5),
         "api_sparse_attention_func_ms": round(api_ms, 5),
-        "roofline_attn": {"kernel": "attn_fwd_kernel (packed mask)", "bound": "mfma", "achieved": round(attn_tflops, 2),
+        "roofline_attn": {"kernel": "attn_fwd_kernel (packed mask" + (", tile map)" if tmap is not None else ")"),
+                          "bound": "mfma", "achieved": round(attn_tflops, 2),
                           "peak": harness.MI355X_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
                           "frac": round(attn_tflops / harness.MI355X_MFMA_F16_TFLOPS, 4),
+                          "frac_cold": round(w.dense_flops / (attn_cold_ms * 1e-3) / 1e12 / harness.MI355X_MFMA_F16_TFLOPS, 4),
+                          "hbm_gbps": round(w.attn_bytes / (attn_ms * 1e-3) / 1e9, 1),
+                          "hbm_frac": round(w.attn_bytes / (attn_ms * 1e-3) / 1e9 / harness.MI355X_HBM_GBPS, 4),
+                          "hbm_frac_cold": round(w.attn_bytes / (attn_cold_ms * 1e-3) / 1e9 / harness.MI355X_HBM_GBPS, 4),
                           "traffic": measured_traffic(w.name, "attn_fwd_kernel"), "algorithmic_bytes": w.attn_bytes},
         "roofline_pack": {"kernel": "pack_flat_kernel" if w.N % 32 == 0 else ("pack_row_kernel" if w.N >= 8 else "pack_short_rows_kernel"),
                           "bound": "hbm", "achieved": round(pack_gbps, 1), "peak": harness.MI355X_HBM_GBPS,
                           "unit": "GB/s", "frac": round(pack_gbps / harness.MI355X_HBM_GBPS, 4),
+                          "frac_cold": round(w.pack_bytes / (pack_cold_ms * 1e-3) / 1e9 / harness.MI355X_HBM_GBPS, 4),
+                          "cache_note": "frac: same mask every launch (last-level cache warm); frac_cold: HBM",
                           "traffic": measured_traffic(w.name, "pack_mask_kernel"), "algorithmic_bytes": w.pack_bytes},
         "roofline_bwd": {"kernel": "attn_bwd_dq_kernel + attn_bwd_dkv_kernel", "bound": "mfma",
                          "achieved": round(bwd_tflops, 2), "peak": harness.MI355X_MFMA_F16_TFLOPS,
@@ -220,26 +289,54 @@ def main():
         gbps = w.fused_bytes / (fused_ms * 1e-3) / 1e9
         tfl = w.dense_flops / (fused_ms * 1e-3) / 1e12
         result["fused_kernel_ms"] = round(fused_ms, 5)
-        result["roofline"] = {"kernel": "attn_fwd_kernel (boolean mask in)", "bound": "hbm", "achieved": round(gbps, 1),
-                              "peak": harness.MI355X_HBM_GBPS, "unit": "GB/s",
-                              "frac": round(gbps / harness.MI355X_HBM_GBPS, 4),
+        cold_gbps = w.fused_bytes / (fused_cold_ms * 1e-3) / 1e9
+        cold_tfl = w.dense_flops / (fused_cold_ms * 1e-3) / 1e12
+        result["fused_kernel_cold_ms"] = round(fused_cold_ms, 5)
+        result["roofline"] = {"kernel": "attn_fwd_kernel (boolean mask in)", "bound": "mfma", "achieved": round(tfl, 2),
+                              "peak": harness.MI355X_MFMA_F16_TFLOPS, "unit": "TFLOP/s",
+                              "frac": round(tfl / harness.MI355X_MFMA_F16_TFLOPS, 4),
+                              "frac_cold": round(cold_tfl / harness.MI355X_MFMA_F16_TFLOPS, 4),
                               "traffic": measured_traffic(w.name, "attn_fwd_bool_mask_kernel"),
                               "algorithmic_bytes": w.fused_bytes,
                               "flop_per_byte": round(w.dense_flops / w.fused_bytes, 1),
-                              "mfma_tflops": round(tfl, 2),
-                              "mfma_frac": round(tfl / harness.MI355X_MFMA_F16_TFLOPS, 4)}
+                              "hbm_gbps": round(gbps, 1),
+                              "hbm_frac": round(gbps / harness.MI355X_HBM_GBPS, 4),
+                              "hbm_frac_cold": round(cold_gbps / harness.MI355X_HBM_GBPS, 4),
+                              "cache_note": "frac / hbm_frac: same tensors every launch, working set inside the 256 MB "
+                                            "last-level cache (the reference's protocol); *_cold: rotating copies, "
+                                            "every launch reads from HBM"}
     else:
         result["roofline"] = dict(result["roofline_attn"])
 
     if not args.no_cpu_baseline:
         from oracle import sma_oracle
+        import numpy as np
         threads = torch.get_num_threads()
         sec = sma_oracle.time_cpu_reference(q.float(), k.float(), v.float(), mask, reps=3)
+        # the input dtype as it is (what the reference's run.py:461 times as "PyTorch Ref")
+        sec_native = sma_oracle.time_cpu_reference(q, k, v, mask, reps=3)
+        # the CPU bit-packer: numpy.packbits(bitorder="little") on the whole mask
+        m_np = mask.numpy()
+        ts = []
+        for _ in range(4):
+            t0 = time.perf_counter()
+            sma_oracle.pack_mask_ref(m_np)
+            ts.append(time.perf_counter() - t0)
+        sec_pack = sorted(ts[1:])[1]
         result["cpu_baseline"] = {
             "value": round(w.dense_flops / sec / 1e12, 5), "unit": "TFLOP/s", "cores": threads,
-            "kind": "port", "ms": round(sec * 1e3, 2),
+            "kind": "port", "ms": round(sec * 1e3, 2), "cpu": cpu_model(),
             "sample": f"whole {w.name} workload, fp32 PyTorch formulation of the oracle on the host CPU, "
-                      f"median of 3 after 1 warm-up, torch threads={threads}, os.cpu_count()={os.cpu_count()}"}
+                      f"median of 3 after 1 warm-up, torch threads={threads}, os.cpu_count()={os.cpu_count()}",
+            "variants": {
+                "native_dtype": {"value": round(w.dense_flops / sec_native / 1e12, 5), "unit": "TFLOP/s",
+                                 "ms": round(sec_native * 1e3, 2), "cores": threads,
+                                 "sample": f"the same in the inputs' own dtype ({'fp16' if w.dtype == torch.float16 else 'bf16'}), "
+                                           "whole workload, median of 3"},
+                "pack_mask": {"value": round(w.pack_bytes / sec_pack / 1e9, 3), "unit": "GB/s",
+                              "ms": round(sec_pack * 1e3, 2), "cores": 1,
+                              "sample": "numpy.packbits(bitorder='little') of the whole mask (the oracle's packer), "
+                                        "median of 3 after 1 warm-up, one thread"}}}
     print(json.dumps(result), flush=True)
 
 
