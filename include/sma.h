@@ -151,7 +151,8 @@ int sma_attn_bwd_static_ws(const void *dout, const void *q, const void *k, const
  * row are contiguous (stride 1, not stored).  Every stride must be >= 0 and a multiple of 8 (rows
  * stay 16-byte aligned); stride_n < 2^23, (N-1)*stride_n*2 + 2*D < 2^31 (bytes inside one (b,h)
  * slab) and stride_b, stride_h < 2^35.  A stride of 0 on
- * an input repeats the same data; the rows of an output must not overlap.
+ * an input repeats the same data; the rows of an output must not overlap (an output with a row
+ * stride below D, or with a zero stride over an extent above 1, is refused with SMA_ERR_STRIDE).
  *
  * Replaces: the twelve stride fields of SparseAttentionParams (stride_qb .. stride_on,
  *           csrc/sparse_attention.h:30-33), which the reference declares and never reads.

@@ -130,23 +130,23 @@ __device__ __forceinline__ u32x2 lds_read_tr16_b64(uint32_t addr) {
 // kernel waits for them explicitly with s_waitcnt vmcnt(n) (completion is in issue order).
 __device__ __forceinline__ void async_copy_b128(uint32_t lds_base, const void *base, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds_base), "v"(voff), "s"(base) : "memory");
+                 :: "s"(lds_base), "v"(voff), "s"(base) : "memory", "m0");
 }
 __device__ __forceinline__ void async_copy_b32(uint32_t lds_base, const void *base, uint32_t voff) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-                 :: "s"(lds_base), "v"(voff), "s"(base) : "memory");
+                 :: "s"(lds_base), "v"(voff), "s"(base) : "memory", "m0");
 }
 // The same with the LDS address given as a scalar base plus a compile-time offset: a loop that
 // copies to many fixed places then keeps one base in a scalar register instead of one per place.
 template <int OFF>
 __device__ __forceinline__ void async_copy_b128_at(uint32_t lds_base, const void *base, uint32_t voff) {
     asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :: "s"(lds_base), "v"(voff), "s"(base), "n"(OFF) : "memory", "scc");
+                 :: "s"(lds_base), "v"(voff), "s"(base), "n"(OFF) : "memory", "scc", "m0");
 }
 template <int OFF>
 __device__ __forceinline__ void async_copy_b32_at(uint32_t lds_base, const void *base, uint32_t voff) {
     asm volatile("s_add_u32 m0, %0, %3\n\ts_nop 0\n\tglobal_load_lds_dword %1, %2"
-                 :: "s"(lds_base), "v"(voff), "s"(base), "n"(OFF) : "memory", "scc");
+                 :: "s"(lds_base), "v"(voff), "s"(base), "n"(OFF) : "memory", "scc", "m0");
 }
 #define WAIT_VMCNT(n) asm volatile("s_waitcnt vmcnt(" #n ")" ::: "memory")
 

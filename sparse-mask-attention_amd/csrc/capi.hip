@@ -15,8 +15,10 @@ inline sma_tensor dense(const void *p, int H, int N, int D)
     return sma_tensor{const_cast<void *>(p), (int64_t)H * N * D, (int64_t)N * D, (int64_t)D};
 }
 
-// Checks one strided [B,H,N,D] tensor and converts it; SMA_OK or an error code.
-int to_rows(const sma_tensor *t, int N, int D, sma::Rows *r)
+// Checks one strided [B,H,N,D] tensor and converts it; SMA_OK or an error code.  An output
+// (`written`) must not fold several rows onto one address: a row stride below D or a zero stride
+// over an extent above 1 would make rows or work-groups overwrite each other.
+int to_rows(const sma_tensor *t, int B, int H, int N, int D, bool written, sma::Rows *r)
 {
     if (t == nullptr || t->data == nullptr) return SMA_ERR_NULL_POINTER;
     if (misaligned(t->data, 16)) return SMA_ERR_ALIGNMENT;
@@ -24,6 +26,8 @@ int to_rows(const sma_tensor *t, int N, int D, sma::Rows *r)
     if ((t->stride_b | t->stride_h | t->stride_n) & 7) return SMA_ERR_STRIDE;
     if ((long long)(N - 1) * t->stride_n * 2 + 2 * D >= (1ll << 31)) return SMA_ERR_STRIDE;
     if (t->stride_b >= (1ll << 35) || t->stride_h >= (1ll << 35) || t->stride_n >= (1ll << 23)) return SMA_ERR_STRIDE;
+    if (written && ((N > 1 && t->stride_n < D) || (H > 1 && t->stride_h == 0) || (B > 1 && t->stride_b == 0)))
+        return SMA_ERR_STRIDE;
     r->p = static_cast<uint16_t *>(t->data);
     r->sb8 = (uint32_t)(t->stride_b >> 3);
     r->sh8 = (uint32_t)(t->stride_h >> 3);
@@ -168,7 +172,7 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
     const sma_tensor *in[8] = {dout, q, k, v, out, dq, dk, dv};
     sma::Rows *to[8] = {&a.dout, &a.q, &a.k, &a.v, &a.out, &a.dq, &a.dk, &a.dv};
     for (int i = 0; i < 8; ++i) {
-        const int st = to_rows(in[i], N, D, to[i]);
+        const int st = to_rows(in[i], B, H, N, D, i >= 5, to[i]);
         if (st != SMA_OK) return st;
     }
     a.lse = lse;
@@ -210,7 +214,7 @@ int sma_attn_fwd_map_strided(const sma_tensor *q, const sma_tensor *k, const sma
     const sma_tensor *in[4] = {q, k, v, out};
     sma::Rows *to[4] = {&a.q, &a.k, &a.v, &a.out};
     for (int i = 0; i < 4; ++i) {
-        const int st = to_rows(in[i], N, D, to[i]);
+        const int st = to_rows(in[i], B, H, N, D, i == 3, to[i]);
         if (st != SMA_OK) return st;
     }
     a.mask = sma::PackedMask{mask_packed, mask_stride_b, mask_stride_h};
@@ -278,7 +282,7 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
     const sma_tensor t[4] = {dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D), dense(out, H, N, D)};
     sma::Rows *to[4] = {&a.q, &a.k, &a.v, &a.out};
     for (int i = 0; i < 4; ++i) {
-        const int st = to_rows(&t[i], N, D, to[i]);
+        const int st = to_rows(&t[i], B, H, N, D, i == 3, to[i]);
         if (st != SMA_OK) return st;
     }
     a.mask = sma::PackedMask{reinterpret_cast<const uint32_t *>(mask), mask_stride_b, mask_stride_h};

@@ -74,6 +74,17 @@ def test_argument_validation_needs_no_gpu(capi):
     assert scall(q=None) == _capi.SMA_ERR_NULL_POINTER
     assert scall(B=0) == _capi.SMA_OK
 
+    # an output whose rows would land on each other is refused; the same strides on an input are fine
+    def ocall(out, q=T(0x1000, 4096, 4096, 64), **kw):
+        a = dict(ok_args, **kw)
+        return fs(q, q, q, p, 128, 128, out, None, a["B"], a["H"], a["N"], a["D"], a["scale"], a["dtype"], None)
+
+    assert ocall(T(0x1000, 4096, 4096, 0)) == _capi.SMA_ERR_STRIDE              # every row at the same place
+    assert ocall(T(0x1000, 4096, 4096, 32)) == _capi.SMA_ERR_STRIDE             # rows half on top of each other
+    assert ocall(T(0x1000, 8192, 0, 64), H=2) == _capi.SMA_ERR_STRIDE           # both heads at the same place
+    assert ocall(T(0x1000, 0, 4096, 64), B=2) == _capi.SMA_ERR_STRIDE           # both batch entries at the same place
+    assert ocall(T(0x1000, 0, 0, 64), B=0, q=T(0x1000, 0, 0, 0)) == _capi.SMA_OK    # nothing to write
+
     # forward straight from the boolean mask: limits are reported, not worked around
     fb = capi.sma_attn_fwd_bool_mask
 
