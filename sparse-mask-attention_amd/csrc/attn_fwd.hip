@@ -30,9 +30,11 @@
 //                 one extra MFMA whose B operand holds -r split into four 16-bit terms and whose
 //                 A operand is all ones.  The accumulator then holds log2 of the unnormalised
 //                 probability: the per-score VALU work is exp2, pack, row-sum and row-max only.
-//   reference r = the online softmax does not track the exact running maximum.  r moves (and O, l
-//                 are rescaled) only when a row's scores leave the window [r-8, r+8] upwards, or
-//                 when its first finite score lies below the window; probabilities stay <= 2^8.
+//   reference r = the online softmax does not track the running maximum.  r moves (and O, l are
+//                 rescaled) only when a row's scores leave the window [r-8, r+8] upwards, or when its
+//                 first kept score lies below the window.  The row maximum of a tile is not even
+//                 computed unless a row meets its first kept key there or the sum of the tile's
+//                 weights shows, afterwards, that a score has run away (then they are redone).
 //   skipping    = with a tile map (one "some bit set" and one "all bits set" bit per 128 x 64 block
 //                 of the mask, made by the packer) the work-group visits only the key tiles that
 //                 hold a set bit for its rows: no copies, no barrier for the others; a block whose
@@ -56,6 +58,7 @@ constexpr int BN = 64;             // keys per tile
 constexpr int NTHREADS = 256;
 constexpr int TILE_BYTES = BN * HD * 2;          // 8 KiB, rows of 128 B
 constexpr float WINDOW_LOG2 = 8.0f;
+constexpr float SUM_LIMIT = 16384.0f;     // a lane's 32 weights of a tile sum to more: some score is far above the window
 
 // Head dims (HDIM) other than 64 reuse the 64-column LDS tile with its 128-byte rows, swizzles and
 // read patterns:
@@ -419,7 +422,8 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
 #pragma unroll
         for (int i = 0; i < 16; ++i) oacc[b][i] = 0.f;
     float ref = 0.f;                    // reference point r, in accumulator units (log2 / pm)
-    float rmax = -__builtin_inff();     // largest score seen so far minus r; -inf = none yet
+    float rmax = -__builtin_inff();     // largest score seen when the maximum was last taken, minus r; -inf = no kept key yet
+    bool all_seen = false;              // wave-uniform: every row of this wavefront has met a kept key
     float l_run = 0.f;                  // this lane's share of sum exp2(pm * (score - r))
     u32x4 refb = {0u, 0u, 0u, 0u};      // -r as four 16-bit terms (lane half 0 only), B operand
     bool ref_used = false;              // false while r == 0 for every row: the extra MFMA is skipped
@@ -469,52 +473,76 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
             sacc[0] = E::mfma(lds_read_b128(ka), qf[s], sacc[0]);
             sacc[1] = E::mfma(lds_read_b128(ka + 4096), qf[s], sacc[1]);
         }
-        // ---- row max over this tile; move the reference only when the window is left ----
-        float mx = -__builtin_inff();
+        // ---- the row maximum of the tile is taken only when it can matter ----
+        // Moves the reference point when a row's scores leave the window [r-8, r+8] upwards, or when
+        // the first kept score of a row lies below it.
+        auto recentre = [&]() __attribute__((always_inline)) {
+            float mx = -__builtin_inff();
 #pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
+            for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
-            for (int i = 0; i < 16; ++i) mx = __builtin_fmaxf(mx, sacc[blk][i]);
-        mx = xhalf_max(mx);
-        const float mxs = POSTMUL ? mx * pm : mx;
-        const bool first = (rmax == -__builtin_inff());
-        const bool move = (mxs > WINDOW_LOG2) | (first & (mxs < -WINDOW_LOG2) & (mx > -__builtin_inff()));
-        const float top = __builtin_fmaxf(rmax, mx);
-        if (__builtin_amdgcn_ballot_w64(move) != 0ull) {
-            // every row of the wavefront re-centres on its own largest score so far
-            const bool any = top > -__builtin_inff();
-            const float new_ref = set_ref(any ? ref + top : ref);
-            const float delta = ref - new_ref;                       // ~ -top
-            const float alpha = first ? 1.0f : __builtin_amdgcn_exp2f(POSTMUL ? delta * pm : delta);
-            ref = new_ref;
-            ref_used = true;
-            l_run *= alpha;
+                for (int i = 0; i < 16; ++i) mx = __builtin_fmaxf(mx, sacc[blk][i]);
+            mx = xhalf_max(mx);
+            const float mxs = POSTMUL ? mx * pm : mx;
+            const bool first = (rmax == -__builtin_inff());
+            const bool move = (mxs > WINDOW_LOG2) | (first & (mxs < -WINDOW_LOG2) & (mx > -__builtin_inff()));
+            const float top = __builtin_fmaxf(rmax, mx);
+            if (__builtin_amdgcn_ballot_w64(move) != 0ull) {
+                // every row of the wavefront re-centres on its own largest score so far
+                const bool any = top > -__builtin_inff();
+                const float new_ref = set_ref(any ? ref + top : ref);
+                const float delta = ref - new_ref;                       // ~ -top
+                const float alpha = first ? 1.0f : __builtin_amdgcn_exp2f(POSTMUL ? delta * pm : delta);
+                ref = new_ref;
+                ref_used = true;
+                l_run *= alpha;
 #pragma unroll
-            for (int i = 0; i < 16; ++i) {
+                for (int i = 0; i < 16; ++i) {
 #pragma unroll
-                for (int b = 0; b < OB; ++b) oacc[b][i] *= alpha;
-                sacc[0][i] += delta; sacc[1][i] += delta;
-            }
-            rmax = top + delta;
-        } else {
-            rmax = top;
-        }
-        // ---- probabilities, packed as the B operands of the PV product ----
-        uint32_t pb[2][2][4];
-        float lsum = 0.f;
-#pragma unroll
-        for (int blk = 0; blk < 2; ++blk)
-#pragma unroll
-            for (int u = 0; u < 2; ++u)
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const float s0 = sacc[blk][8 * u + 2 * i], s1 = sacc[blk][8 * u + 2 * i + 1];
-                    const float p0 = __builtin_amdgcn_exp2f(POSTMUL ? s0 * pm : s0);
-                    const float p1 = __builtin_amdgcn_exp2f(POSTMUL ? s1 * pm : s1);
-                    const uint32_t pk = E::pack2_prob(p0, p1);
-                    pb[blk][u][i] = pk;
-                    lsum = E::add2(pk, lsum);
+                    for (int b = 0; b < OB; ++b) oacc[b][i] *= alpha;
+                    sacc[0][i] += delta; sacc[1][i] += delta;
                 }
+                rmax = top + delta;
+            } else {
+                rmax = top;
+            }
+        };
+        // probabilities, packed as the B operands of the PV product; returns this lane's sum of them
+        uint32_t pb[2][2][4];
+        auto exponentials = [&]() __attribute__((always_inline)) -> float {
+            float lsum = 0.f;
+#pragma unroll
+            for (int blk = 0; blk < 2; ++blk)
+#pragma unroll
+                for (int u = 0; u < 2; ++u)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const float s0 = sacc[blk][8 * u + 2 * i], s1 = sacc[blk][8 * u + 2 * i + 1];
+                        const float p0 = __builtin_amdgcn_exp2f(POSTMUL ? s0 * pm : s0);
+                        const float p1 = __builtin_amdgcn_exp2f(POSTMUL ? s1 * pm : s1);
+                        const uint32_t pk = E::pack2_prob(p0, p1);
+                        pb[blk][u][i] = pk;
+                        lsum = E::add2(pk, lsum);
+                    }
+            return lsum;
+        };
+        // A row needs the maximum when it meets its first kept key (to choose its reference point)
+        // and when a score runs away above the window.  The first is known beforehand; the second
+        // shows afterwards, in the sum of the exponentials (needed anyway): a weight above 2^14, an
+        // infinity or a NaN makes a lane's sum of 32 weights exceed SUM_LIMIT, and no weight that
+        // the window would have let pass (<= 2^8) can.  Only then are the maximum taken, the
+        // reference moved and the exponentials redone.
+        bool with_max = false;
+        if (!all_seen) with_max = __builtin_amdgcn_ballot_w64((rmax == -__builtin_inff()) & ((w2.x | w2.y) != 0u)) != 0ull;
+        if (with_max) {
+            recentre();
+            all_seen = __builtin_amdgcn_ballot_w64(rmax == -__builtin_inff()) == 0ull;
+        }
+        float lsum = exponentials();
+        if (!with_max && __builtin_amdgcn_ballot_w64(!(lsum <= SUM_LIMIT)) != 0ull) {
+            recentre();
+            lsum = exponentials();
+        }
         l_run += lsum;
         // ---- O^T += V^T * P^T : oacc[b][4g+j] = out(query l32, d = 32b + 8g + 4hh + j) ----
 #pragma unroll

@@ -92,3 +92,42 @@ def test_row_maximum_at_the_edge_of_the_window(dev, dtype, top_log2):
     assert torch.equal(fused, out)
     lse_ref = O.lse_ref(q.float(), k.float(), mask)
     assert torch.allclose(lse.cpu(), lse_ref, atol=2e-2, rtol=0)
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("step", [3.0, 12.0, 40.0, 200.0])
+def test_scores_that_climb_from_tile_to_tile(dev, dtype, step):
+    """The largest score of every row grows by `step` (log2 units of the weight) with each tile of 64
+    keys, so that the kernel, which takes a row maximum only when the sum of a tile's weights tells
+    it to, has to notice again and again (small steps stay inside what it tolerates for a while,
+    large ones overflow the exponential itself).  Some rows meet their first kept key only in a
+    late tile."""
+    N, D = 448, 64
+    g = torch.Generator().manual_seed(int(step))
+    ln2 = math.log(2.0)
+    q = torch.zeros(1, 2, N, D)
+    q[..., 0] = 8.0                                              # (q . k) / sqrt(D) = k[0]
+    k = torch.randn(1, 2, N, D, generator=g) * 0.2
+    k[..., 0] = (torch.arange(N) // 64).float().view(1, 1, N) * step * ln2 + torch.randn(1, 2, N, generator=g)
+    v = torch.randn(1, 2, N, D, generator=g)
+    q, k, v = q.to(dtype), k.to(dtype), v.to(dtype)
+    mask = torch.rand(1, 2, N, N, generator=g) < 0.3
+    late = torch.arange(N) % 5 == 0                              # these rows keep nothing before key 200
+    mask[:, :, late, :200] = False
+    mask[:, :, 7, :] = False                                     # and one keeps nothing at all
+    packed = torch.from_numpy(O.pack_mask_ref(mask)).to(dev)
+    out, lse = _capi.attn_fwd(q.to(dev), k.to(dev), v.to(dev), packed, want_lse=True)
+    fused = _capi.attn_fwd_bool_mask(q.to(dev), k.to(dev), v.to(dev), mask.to(dev))
+    torch.cuda.synchronize()
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    assert torch.isfinite(out.float()).all()
+    err = (out.float().cpu() - ref).abs().max().item()
+    assert torch.allclose(out.float().cpu(), ref, atol=ATOL, rtol=RTOL[dtype]), f"max err {err:.3e}"
+    assert torch.equal(fused, out)
+    assert (out[:, :, 7] == 0).all() and (lse[:, :, 7] == -math.inf).all()
+    lse_ref = O.lse_ref(q.float(), k.float(), mask)
+    fin = torch.isfinite(lse_ref)
+    # q is rounded to its 16-bit format once more after the scale has been folded into it, which
+    # moves every score of a row, and with it lse, by up to half a unit in the last place
+    eps = {torch.float16: 2.0 ** -11, torch.bfloat16: 2.0 ** -8}[dtype]
+    assert torch.allclose(lse.cpu()[fin], lse_ref[fin], atol=2e-2, rtol=eps)
