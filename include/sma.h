@@ -220,6 +220,16 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
                          float *delta_ws, int B, int H, int N, int D, float scale, int dtype,
                          void *stream);
 
+/* Yardstick for the MFMA roofline, used by the benchmark (not by the attention path): launches
+ * `work_groups` work-groups of 12 wavefronts that each issue 8 * iters MFMAs of the kind the
+ * attention kernels use (v_mfma_f32_32x32x16_f16), on operands that are all zero (random_operands
+ * == 0) or random fp16 numbers.  Thread 0 of work-group g leaves in stamps[2g] the shader-clock
+ * ticks and in stamps[2g+1] the 100 MHz ticks that its loop took (stamps: device memory, 2 *
+ * work_groups int64).  Time the launch to get the sustained MFMA rate; the quotient of the two
+ * stamps is the shader clock in units of 100 MHz.  No counterpart in the reference.
+ */
+int sma_probe_mfma_stream(int random_operands, int iters, int work_groups, long long *stamps, void *stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -28,7 +28,7 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 LIB_NAME = "libsma_hip.so"
 MODULE_NAME = "sparse_attn_cuda"
-HIP_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "pack_mask.hip", "capi.hip"]
+HIP_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "pack_mask.hip", "capi.hip", "probe.hip"]
 GPU_ARCH = "gfx950"
 
 

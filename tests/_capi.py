@@ -60,6 +60,8 @@ def load():
         lib.sma_pack_mask_map.argtypes = [vp, vp, vp, ci, ci, ci, vp]
         lib.sma_attn_fwd_map.restype = ci
         lib.sma_attn_fwd_map.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_probe_mfma_stream.restype = ci
+        lib.sma_probe_mfma_stream.argtypes = [ci, ci, ci, vp, vp]
         lib.sma_attn_bwd_static_ws.restype = ci
         lib.sma_attn_bwd_static_ws.argtypes = [vp] * 10 + [ci, ci, ci, ci, cf, ci, vp]
         tp, i64 = ctypes.POINTER(SmaTensor), ctypes.c_int64

@@ -376,3 +376,21 @@ def test_inference_entry_point_reads_the_bool_mask_itself(sa, dev, monkeypatch):
     assert o32.dtype == torch.float32
     ref = O.sparse_attention_ref(q.bfloat16().float(), k.bfloat16().float(), v.bfloat16().float(), mask)
     assert torch.allclose(o32.cpu(), ref, atol=1e-2, rtol=2e-2)
+
+
+def test_mfma_stream_probe_runs_and_reports_a_clock(dev):
+    """The benchmark's yardstick kernel: finishes, and the two tick counts it leaves give a shader
+    clock that a GPU of this kind can have."""
+    import _capi
+    lib = _capi.load()
+    groups = 8
+    stamps = torch.zeros(2 * groups, dtype=torch.int64, device=dev)
+    for random_operands in (0, 1):
+        assert lib.sma_probe_mfma_stream(random_operands, 2000, groups, stamps.data_ptr(), None) == _capi.SMA_OK
+        torch.cuda.synchronize()
+        st = stamps.view(groups, 2).double().cpu()
+        assert (st > 0).all()
+        ghz = (st[:, 0] / (st[:, 1] * 10.0)).mean().item()
+        assert 0.3 < ghz < 3.0, ghz
+    assert lib.sma_probe_mfma_stream(1, 10, 0, None, None) == _capi.SMA_OK
+    assert lib.sma_probe_mfma_stream(1, 10, 4, None, None) == _capi.SMA_ERR_NULL_POINTER
