@@ -200,7 +200,7 @@ def main():
     ext.forward(qd, kd, vd, packed, out, lse, scale, True)
     dout = torch.randn(qd.shape, generator=torch.Generator().manual_seed(43)).to(qd.dtype).to(dev)
     dq, dk, dv = (torch.empty_like(qd) for _ in range(3))
-    bwd_ms = event_time_ms(lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale),
+    bwd_ms = event_time_ms(lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale, tmap),
                            5, reps, torch)
     bwd_tflops = w.bwd_dense_flops / (bwd_ms * 1e-3) / 1e12
 

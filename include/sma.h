@@ -129,6 +129,17 @@ int sma_attn_bwd(const void *dout, const void *q, const void *k, const void *v, 
                  const float *lse, const uint32_t *mask_packed, void *dq, void *dk, void *dv,
                  float *delta_ws, int B, int H, int N, int D, float scale, int dtype, void *stream);
 
+/* sma_attn_bwd with a tile map (see sma_tile_map) of the same packed mask: both kernels visit only
+ * the 64 x 64 blocks in which the mask keeps something.  tile_map == NULL is sma_attn_bwd; the
+ * gradients are the same bit for bit.  sma_attn_bwd_map_strided is the strided form (map
+ * contiguous [Bm,Hm,T,2,TW] with the mask's own Bm, Hm).
+ */
+int sma_attn_bwd_map(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                     const float *lse, const uint32_t *mask_packed, const uint32_t *tile_map, void *dq,
+                     void *dk, void *dv, float *delta_ws, int B, int H, int N, int D, float scale, int dtype,
+                     void *stream);
+
+
 /* sma_attn_bwd without the workspace argument, for callers that cannot allocate device memory at
  * all (code running under HIP graph capture, tight serving loops, harnesses that forbid
  * hipMalloc): the per-row sums that the two kernels exchange live in a fixed array inside the
@@ -219,6 +230,14 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
                          const sma_tensor *dq, const sma_tensor *dk, const sma_tensor *dv,
                          float *delta_ws, int B, int H, int N, int D, float scale, int dtype,
                          void *stream);
+
+/* sma_attn_bwd_map for strided tensors and a shared mask (see sma_attn_bwd_map). */
+int sma_attn_bwd_map_strided(const sma_tensor *dout, const sma_tensor *q, const sma_tensor *k,
+                             const sma_tensor *v, const sma_tensor *out, const float *lse,
+                             const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                             const uint32_t *tile_map, const sma_tensor *dq, const sma_tensor *dk,
+                             const sma_tensor *dv, float *delta_ws, int B, int H, int N, int D, float scale,
+                             int dtype, void *stream);
 
 /* Yardstick for the MFMA roofline, used by the benchmark (not by the attention path): launches
  * `work_groups` work-groups of 12 wavefronts that each issue 8 * iters MFMAs of the kind the

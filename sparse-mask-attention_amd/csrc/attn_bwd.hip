@@ -218,7 +218,31 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_bwd_dq_ker
         issue_tile<NH>(lds0 + st * STAGE_BYTES, kb, a.k.sn, t * BN, N, tc, wave);
         issue_tile<NH>(lds0 + st * STAGE_BYTES + C::OFF_B, vb, a.v.sn, t * BN, N, tc, wave);
     };
-    issue(0, 0);
+    // With a tile map only the key tiles that hold a set mask bit for this work-group's rows are
+    // visited (the map has one row of "live" bits per block of 64 query rows: two of them are ORed);
+    // without one, all.  Wave-uniform walk over the set bits, a word (32 tiles) at a time.
+    const int TW = (T + 31) >> 5;
+    const uint32_t *mapw = nullptr, *mapw2 = nullptr;
+    if (a.tile_map != nullptr) {
+        mapw = a.tile_map + bi * a.map_sb + hi * a.map_sh + (size_t)(2 * qt) * 2 * TW;
+        mapw2 = (2 * qt + 1 < T) ? mapw + 2 * TW : mapw;
+    }
+    int cur_w = -1;
+    uint32_t live_w = 0u;
+    auto next_tile = [&]() __attribute__((always_inline)) -> int {     // next live tile, T if there is none
+        while (live_w == 0u) {
+            if (++cur_w >= TW) return T;
+            uint32_t lv = 0xffffffffu;
+            if (mapw != nullptr) lv = __builtin_amdgcn_readfirstlane(mapw[cur_w] | mapw2[cur_w]);
+            if (cur_w == TW - 1 && (T & 31) != 0) lv &= (1u << (T & 31)) - 1u;
+            live_w = lv;
+        }
+        const int b = __builtin_ctz(live_w);
+        live_w &= live_w - 1u;
+        return 32 * cur_w + b;
+    };
+    const int t_first = next_tile();
+    if (t_first < T) issue(t_first, 0);
     if (tid < 64)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
 
@@ -230,13 +254,15 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_bwd_dq_ker
     const uint32_t lut_addr = lds0 + OFF_LUT;
     const uint32_t nib_shift = 4u - 4u * hh;
 
-    for (int t = 0; t < T; ++t) {
-        const int st = t & 1;
+    int st = 1;
+    for (int t = t_first, t_next; t < T; t = t_next) {
+        t_next = next_tile();
+        st ^= 1;                  // the visits alternate between the two stages
         const uint32_t so = lds0 + st * STAGE_BYTES;
         WAIT_VMCNT(0);
         if (ragged && t == T - 1) zero_tile_tail(so, 2 * NH, t * BN, N, tc, wave, lane);
         __syncthreads();          // tile t of every wave landed; the other stage is free
-        if (t + 1 < T) issue(t + 1, st ^ 1);
+        if (t_next < T) issue(t_next, st ^ 1);
 
         u32x2 w2 = lds_read_b64(lds0 + OFF_AUX + st * AUX_BYTES + wave * 256 + l32 * 8);
         if (t == T - 1) { w2.x &= a.last_mask0; w2.y &= a.last_mask1; }
@@ -380,7 +406,29 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
         issue_tile<NH>(lds0 + st * STAGE_BYTES, qb, a.q.sn, r0, N, tc, wave);
         issue_tile<NH>(lds0 + st * STAGE_BYTES + C::OFF_B, dob, a.dout.sn, r0, N, tc, wave);
     };
-    issue(0, 0);
+    // With a tile map only the blocks of 64 query rows in which the mask keeps something for this
+    // work-group's 128 keys (its two key tiles 2kt, 2kt+1: neighbouring bits of one word of the
+    // row block's "live" bits) are visited: lane r of a wavefront looks at row block 64c + r, a
+    // ballot turns the 64 answers into the bits that are walked.  Every wavefront does the same.
+    const int TW = (T + 31) >> 5;
+    const uint32_t *mapc = a.tile_map != nullptr
+        ? a.tile_map + bi * a.map_sb + hi * a.map_sh + ((2 * kt) >> 5) : nullptr;
+    int cur_c = -1;
+    unsigned long long live_c = 0ull;
+    auto next_tile = [&]() __attribute__((always_inline)) -> int {     // next live row block, T if there is none
+        while (live_c == 0ull) {
+            if (64 * ++cur_c >= T) return T;
+            const int r = 64 * cur_c + lane;
+            bool lv = r < T;
+            if (mapc != nullptr && lv) lv = ((mapc[(size_t)r * 2 * TW] >> ((2 * kt) & 31)) & 3u) != 0u;
+            live_c = __builtin_amdgcn_ballot_w64(lv);
+        }
+        const int b = __builtin_ctzll(live_c);
+        live_c &= live_c - 1ull;
+        return 64 * cur_c + b;
+    };
+    const int t_first = next_tile();
+    if (t_first < T) issue(t_first, 0);
 
     f32x16 dkacc[DK ? OB : 1], dvacc[DV ? OB : 1];      // [2 * half + dblk]: 32 columns each
 #pragma unroll
@@ -393,7 +441,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
 
     // one q tile; the ring stage is a compile-time constant so that every LDS address of the body is
     // a register plus an immediate
-    auto tile = [&](int t, auto st_c) __attribute__((always_inline)) {
+    auto tile = [&](int t, int t_next, auto st_c) __attribute__((always_inline)) {
         constexpr int st = decltype(st_c)::value;
         const uint32_t so = lds0 + st * STAGE_BYTES;
         const uint32_t aux = lds0 + OFF_AUX + st * AUX_BYTES;
@@ -414,7 +462,7 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
         }
         if (ragged && t == T - 1) zero_tile_tail(so, 2 * NH, t * BN, N, tc, wave, lane);
         __syncthreads();
-        if (t + 1 < T) issue(t + 1, st ^ 1);
+        if (t_next < T) issue(t_next, st ^ 1);
         if (!wave_valid) return;
 
 #pragma unroll
@@ -499,9 +547,12 @@ __global__ __launch_bounds__(NTHREADS, 2) void attn_bwd_dkv_kernel(const AttnBwd
             }
         }
     };
-    for (int t = 0; t < T; t += 2) {
-        tile(t, std::integral_constant<int, 0>{});
-        if (t + 1 < T) tile(t + 1, std::integral_constant<int, 1>{});
+    for (int t = t_first; t < T;) {
+        const int tn = next_tile();
+        tile(t, tn, std::integral_constant<int, 0>{});
+        if (tn >= T) break;
+        t = next_tile();
+        tile(tn, t, std::integral_constant<int, 1>{});
     }
     WAIT_VMCNT(0);
     __syncthreads();

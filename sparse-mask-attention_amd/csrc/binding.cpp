@@ -9,7 +9,7 @@
 //   tile_map(mask_packed) -> int32 Tensor [B, H, ceil(N/64), 2, ceil(ceil(N/64)/32)]   (not in the
 //       reference: which 64 x 64 blocks of the mask hold a set bit / nothing but set bits; passed to
 //       `forward` as tile_map, key tiles without a set bit are neither loaded nor computed)
-//   backward(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, scale) -> None   (called by the
+//   backward(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, scale, tile_map=None) -> None   (called by the
 //       reference's Python API, python/sparse_attention.py:91-94, but absent from its binding)
 //   forward_bool_mask(q, k, v, mask, out, lse, scale, is_training, packed_out=None) -> None   (not in
 //       the reference: `forward` with the boolean mask itself in place of the packed one, one launch
@@ -70,6 +70,20 @@ void mask_strides(const torch::Tensor &mp, const torch::Tensor &q, int64_t *sb, 
     *sh = mp.size(1) == 1 ? 0 : N * nw;
 }
 
+// The optional tile map of mask_packed ([Bm, Hm, T, 2, ceil(T/32)] int32, T = ceil(N/64)), checked; nullptr if absent.
+const uint32_t *map_pointer(const c10::optional<torch::Tensor> &tile_map, const torch::Tensor &mask_packed,
+                            const torch::Tensor &q)
+{
+    if (!tile_map.has_value() || !tile_map->defined()) return nullptr;
+    const torch::Tensor &m = *tile_map;
+    const int64_t T = (q.size(2) + 63) / 64;
+    TORCH_CHECK(m.device() == q.device() && m.scalar_type() == at::kInt && m.dim() == 5 &&
+                    m.size(0) == mask_packed.size(0) && m.size(1) == mask_packed.size(1) && m.size(2) == T &&
+                    m.size(3) == 2 && m.size(4) == (T + 31) / 32 && m.is_contiguous(),
+                "tile_map must be the contiguous int32 result of tile_map(mask_packed)");
+    return reinterpret_cast<const uint32_t *>(m.data_ptr<int32_t>());
+}
+
 void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,
              const torch::Tensor &mask_packed, torch::Tensor out,
              const c10::optional<torch::Tensor> &lse, double scale, bool is_training,
@@ -99,16 +113,7 @@ void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor
         lse_ptr = lse->data_ptr<float>();
     }
     TORCH_CHECK(B <= INT32_MAX && H <= INT32_MAX && N <= INT32_MAX, "extent too large");
-    const uint32_t *map_ptr = nullptr;
-    if (tile_map.has_value() && tile_map->defined()) {
-        const torch::Tensor &m = *tile_map;
-        const int64_t T = (N + 63) / 64;
-        TORCH_CHECK(m.device() == q.device() && m.scalar_type() == at::kInt && m.dim() == 5 &&
-                        m.size(0) == mask_packed.size(0) && m.size(1) == mask_packed.size(1) && m.size(2) == T &&
-                        m.size(3) == 2 && m.size(4) == (T + 31) / 32 && m.is_contiguous(),
-                    "tile_map must be the contiguous int32 result of tile_map(mask_packed)");
-        map_ptr = reinterpret_cast<const uint32_t *>(m.data_ptr<int32_t>());
-    }
+    const uint32_t *map_ptr = map_pointer(tile_map, mask_packed, q);
 
     const c10::DeviceGuard guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
@@ -192,7 +197,7 @@ void forward_bool_mask(const torch::Tensor &q, const torch::Tensor &k, const tor
 void backward(const torch::Tensor &dout, const torch::Tensor &q, const torch::Tensor &k,
               const torch::Tensor &v, const torch::Tensor &out, const torch::Tensor &lse,
               const torch::Tensor &mask_packed, torch::Tensor dq, torch::Tensor dk,
-              torch::Tensor dv, double scale)
+              torch::Tensor dv, double scale, const c10::optional<torch::Tensor> &tile_map)
 {
     TORCH_CHECK(q.is_cuda(), "q must be a GPU tensor");
     TORCH_CHECK(q.dim() == 4, "q must be 4D [B, H, N, D]");
@@ -217,15 +222,17 @@ void backward(const torch::Tensor &dout, const torch::Tensor &q, const torch::Te
                 "lse must be a contiguous float32 [B, H, N] tensor on q's device");
     TORCH_CHECK(B <= INT32_MAX && H <= INT32_MAX && N <= INT32_MAX, "extent too large");
 
+    const uint32_t *map_ptr = map_pointer(tile_map, mask_packed, q);
+
     const c10::DeviceGuard guard(q.device());
     torch::Tensor delta = torch::empty({B, H, N}, lse.options());      // workspace of the C entry point
     hipStream_t stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
-    const int st = sma_attn_bwd_strided(&d[0], &d[1], &d[2], &d[3], &d[4], lse.data_ptr<float>(),
-                                        reinterpret_cast<const uint32_t *>(mask_packed.data_ptr<int32_t>()),
-                                        msb, msh, &d[5], &d[6], &d[7], delta.data_ptr<float>(), (int)B, (int)H,
-                                        (int)N, (int)D, (float)scale,
-                                        dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
-    check_status(st, "sma_attn_bwd_strided");
+    const int st = sma_attn_bwd_map_strided(&d[0], &d[1], &d[2], &d[3], &d[4], lse.data_ptr<float>(),
+                                            reinterpret_cast<const uint32_t *>(mask_packed.data_ptr<int32_t>()),
+                                            msb, msh, map_ptr, &d[5], &d[6], &d[7], delta.data_ptr<float>(), (int)B,
+                                            (int)H, (int)N, (int)D, (float)scale,
+                                            dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
+    check_status(st, "sma_attn_bwd_map_strided");
 }
 
 torch::Tensor pack_mask(const torch::Tensor &mask)
@@ -281,7 +288,8 @@ PYBIND11_MODULE(sparse_attn_cuda, m)
           py::arg("mask_packed"));
     m.def("backward", &backward, "Sparse-mask attention backward (dq, dk, dv are overwritten)",
           py::arg("dout"), py::arg("q"), py::arg("k"), py::arg("v"), py::arg("out"), py::arg("lse"),
-          py::arg("mask_packed"), py::arg("dq"), py::arg("dk"), py::arg("dv"), py::arg("scale"));
+          py::arg("mask_packed"), py::arg("dq"), py::arg("dk"), py::arg("dv"), py::arg("scale"),
+          py::arg("tile_map") = py::none());
     m.def("forward_bool_mask", &forward_bool_mask,
           "Sparse-mask attention forward straight from the bool mask (one launch; see bool_mask_supported)",
           py::arg("q"), py::arg("k"), py::arg("v"), py::arg("mask"), py::arg("out"), py::arg("lse"),

@@ -147,12 +147,12 @@ static void last_tile_masks(int N, uint32_t *m0, uint32_t *m1)
     *m1 = v1 >= 32 ? 0xffffffffu : ((1u << v1) - 1u);
 }
 
-int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_tensor *k,
-                         const sma_tensor *v, const sma_tensor *out, const float *lse,
-                         const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
-                         const sma_tensor *dq, const sma_tensor *dk, const sma_tensor *dv,
-                         float *delta_ws, int B, int H, int N, int D, float scale, int dtype,
-                         void *stream)
+int sma_attn_bwd_map_strided(const sma_tensor *dout, const sma_tensor *q, const sma_tensor *k,
+                             const sma_tensor *v, const sma_tensor *out, const float *lse,
+                             const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                             const uint32_t *tile_map, const sma_tensor *dq, const sma_tensor *dk,
+                             const sma_tensor *dv, float *delta_ws, int B, int H, int N, int D, float scale,
+                             int dtype, void *stream)
 {
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
     if (D != 32 && D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
@@ -165,7 +165,9 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
     // a lane's byte offset into the packed mask of one (b,h) is a 32-bit register
     if ((long long)N * ((N + 31) / 32) * 4 >= (1ll << 32)) return SMA_ERR_BAD_SHAPE;
-    if (misaligned(mask_packed, 4) || misaligned(lse, 4) || misaligned(delta_ws, 4)) return SMA_ERR_ALIGNMENT;
+    if (misaligned(mask_packed, 4) || misaligned(lse, 4) || misaligned(delta_ws, 4) || (tile_map && misaligned(tile_map, 4)))
+        return SMA_ERR_ALIGNMENT;
+    if (tile_map && N > 131072) return SMA_ERR_BAD_SHAPE;
     if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 
     sma::AttnBwdArgs a;
@@ -178,6 +180,10 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
     a.lse = lse;
     a.mask = sma::PackedMask{mask_packed, mask_stride_b, mask_stride_h};
     a.delta = delta_ws;
+    a.tile_map = tile_map;
+    const long long map_words = sma_tile_map_words(N);
+    a.map_sh = (H > 1 && mask_stride_h != 0) ? map_words : 0;
+    a.map_sb = (B > 1 && mask_stride_b != 0) ? ((H > 1 && mask_stride_h != 0) ? (long long)H : 1ll) * map_words : 0;
     a.BH = (int)BH;
     a.H = H;
     a.N = N;
@@ -188,6 +194,29 @@ int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_
     last_tile_masks(N, &a.last_mask0, &a.last_mask1);
     const hipError_t e = sma::launch_attn_bwd(a, dtype == SMA_DTYPE_BF16, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
+}
+
+int sma_attn_bwd_strided(const sma_tensor *dout, const sma_tensor *q, const sma_tensor *k,
+                         const sma_tensor *v, const sma_tensor *out, const float *lse,
+                         const uint32_t *mask_packed, int64_t mask_stride_b, int64_t mask_stride_h,
+                         const sma_tensor *dq, const sma_tensor *dk, const sma_tensor *dv,
+                         float *delta_ws, int B, int H, int N, int D, float scale, int dtype,
+                         void *stream)
+{
+    return sma_attn_bwd_map_strided(dout, q, k, v, out, lse, mask_packed, mask_stride_b, mask_stride_h, nullptr, dq,
+                                    dk, dv, delta_ws, B, H, N, D, scale, dtype, stream);
+}
+
+int sma_attn_bwd_map(const void *dout, const void *q, const void *k, const void *v, const void *out,
+                     const float *lse, const uint32_t *mask_packed, const uint32_t *tile_map, void *dq,
+                     void *dk, void *dv, float *delta_ws, int B, int H, int N, int D, float scale, int dtype,
+                     void *stream)
+{
+    const sma_tensor t[8] = {dense(dout, H, N, D), dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D),
+                             dense(out, H, N, D), dense(dq, H, N, D), dense(dk, H, N, D), dense(dv, H, N, D)};
+    const int64_t msh = (int64_t)N * ((N + 31) / 32);
+    return sma_attn_bwd_map_strided(&t[0], &t[1], &t[2], &t[3], &t[4], lse, mask_packed, msh * H, msh, tile_map,
+                                    &t[5], &t[6], &t[7], delta_ws, B, H, N, D, scale, dtype, stream);
 }
 
 int sma_attn_fwd_map_strided(const sma_tensor *q, const sma_tensor *k, const sma_tensor *v,

@@ -79,6 +79,8 @@ struct AttnBwdArgs {
     PackedMask mask;
     Rows dq, dk, dv;
     float *delta;                              // [BH, N] workspace: sum_d dout * out per query row
+    const uint32_t *tile_map;                  // nullptr, or the tile map of the mask (as in AttnArgs)
+    long long map_sb, map_sh;
     int BH, H, N;
     int D;                                     // head dim: 32, 64 or 128
     int qtiles;                                // ceil(N / 128)

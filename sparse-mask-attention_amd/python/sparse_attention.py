@@ -133,6 +133,7 @@ class SparseAttentionFunction(Function):
         sparse_attn_cuda.forward(q, k, v, mask_packed, out, lse, scale, True, tile_map)
         ctx.save_for_backward(q, k, v, out, lse, mask_packed)
         ctx.scale = scale
+        ctx.tile_map = tile_map
         return out
 
     @staticmethod
@@ -141,7 +142,7 @@ class SparseAttentionFunction(Function):
         dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
         # the call the reference makes at python/sparse_attention.py:91-94
         sparse_attn_cuda.backward(_rows(dout.to(q.dtype)), q, k, v, out, lse, mask_packed,
-                                  dq, dk, dv, ctx.scale)
+                                  dq, dk, dv, ctx.scale, getattr(ctx, "tile_map", None))
         return dq, dk, dv, None, None, None, None, None
 
 

@@ -62,6 +62,8 @@ def load():
         lib.sma_attn_fwd_map.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_probe_mfma_stream.restype = ci
         lib.sma_probe_mfma_stream.argtypes = [ci, ci, ci, vp, vp]
+        lib.sma_attn_bwd_map.restype = ci
+        lib.sma_attn_bwd_map.argtypes = [vp] * 12 + [ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_bwd_static_ws.restype = ci
         lib.sma_attn_bwd_static_ws.argtypes = [vp] * 10 + [ci, ci, ci, ci, cf, ci, vp]
         tp, i64 = ctypes.POINTER(SmaTensor), ctypes.c_int64
@@ -71,6 +73,8 @@ def load():
         lib.sma_attn_bwd_strided.argtypes = [tp] * 5 + [vp, vp, i64, i64, tp, tp, tp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_fwd_map_strided.restype = ci
         lib.sma_attn_fwd_map_strided.argtypes = [tp, tp, tp, vp, i64, i64, vp, tp, vp, ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_attn_bwd_map_strided.restype = ci
+        lib.sma_attn_bwd_map_strided.argtypes = [tp] * 5 + [vp, vp, i64, i64, vp, tp, tp, tp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_fwd_bool_mask.restype = ci
         lib.sma_attn_fwd_bool_mask.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         _lib = lib
@@ -187,6 +191,23 @@ def attn_bwd(dout, q, k, v, out, lse, packed, scale=None):
                           delta.data_ptr(), B, H, N, D, scale, dt, _stream())
     assert st == SMA_OK, lib.sma_strerror(st)
     return dq, dk, dv, delta
+
+
+def attn_bwd_map(dout, q, k, v, out, lse, packed, tm, scale=None):
+    """Backward through sma_attn_bwd_map (tile map of the same mask); returns (dq, dk, dv)."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    dq, dk, dv = (torch.full_like(q, float("nan")) for _ in range(3))
+    delta = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device)
+    st = lib.sma_attn_bwd_map(dout.data_ptr(), q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(),
+                              lse.data_ptr(), packed.data_ptr(), tm.data_ptr() if tm is not None else None,
+                              dq.data_ptr(), dk.data_ptr(), dv.data_ptr(), delta.data_ptr(), B, H, N, D, scale, dt,
+                              _stream())
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return dq, dk, dv
 
 
 def attn_bwd_static_ws(dout, q, k, v, out, lse, packed, scale=None, expect=SMA_OK):

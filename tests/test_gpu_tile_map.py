@@ -89,6 +89,39 @@ def test_forward_with_map_equals_forward_without(dev, N, D, dtype):
         assert torch.allclose(got.float().cpu(), ref, atol=1e-2, rtol=rtol), (name, N, D, dtype)
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("N", [64, 200, 333, 512])
+def test_backward_with_map_equals_backward_without(dev, N, D, dtype):
+    g = torch.Generator().manual_seed(7000 * D + N)
+    q, k, v, do = (torch.randn(2, 2, N, D, generator=g).to(dtype).to(dev) for _ in range(4))
+    for name, mask in _masks(N, g):
+        B, H = mask.shape[:2]
+        packed, tm = _capi.pack_mask_map(mask.to(dev))
+        qq, kk, vv, dd = q[:B], k[:B], v[:B], do[:B]
+        out, lse = _capi.attn_fwd(qq, kk, vv, packed, want_lse=True)
+        want = _capi.attn_bwd(dd, qq, kk, vv, out, lse, packed)[:3]
+        got = _capi.attn_bwd_map(dd, qq, kk, vv, out, lse, packed, tm)
+        torch.cuda.synchronize()
+        for gname, a, b in zip(("dq", "dk", "dv"), got, want):
+            assert torch.equal(a, b), (gname, name, N, D, dtype)
+
+
+def test_backward_with_map_and_more_than_64_row_blocks(dev):
+    N = 64 * 66 + 3
+    g = torch.Generator().manual_seed(2)
+    mask = torch.rand(1, 1, N, N, generator=g) < 0.0003
+    mask[0, 0, 64 * 65:, :100] = True
+    q, k, v, do = (torch.randn(1, 1, N, 64, generator=g).half().to(dev) for _ in range(4))
+    packed, tm = _capi.pack_mask_map(mask.to(dev))
+    out, lse = _capi.attn_fwd_map(q, k, v, packed, tm, want_lse=True)
+    want = _capi.attn_bwd(do, q, k, v, out, lse, packed)[:3]
+    got = _capi.attn_bwd_map(do, q, k, v, out, lse, packed, tm)
+    torch.cuda.synchronize()
+    for a, b in zip(got, want):
+        assert torch.equal(a, b)
+
+
 def test_shared_mask_and_strided_tensors(dev):
     g = torch.Generator().manual_seed(3)
     B, H, N = 3, 4, 300
@@ -154,6 +187,10 @@ def test_python_api_with_tile_map(dev):
     out.sum().backward()
     torch.cuda.synchronize()
     assert all(torch.isfinite(t.grad.float()).all() and t.grad.abs().sum() > 0 for t in leaves)
+    plain = [t.clone().requires_grad_(True) for t in (q, k, v)]
+    sa.sparse_attention(*plain, None, mask_packed=packed).sum().backward()
+    torch.cuda.synchronize()
+    assert all(torch.equal(a.grad, b.grad) for a, b in zip(leaves, plain))     # the backward walked the map too
     with pytest.raises(AssertionError):
         sa.sparse_attention_func(q, k, v, mask, tile_map=tm)          # a map without its packed mask
     with pytest.raises(RuntimeError):
