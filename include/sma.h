@@ -221,6 +221,23 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
                            uint32_t *packed_out, int B, int H, int N, int D, float scale, int dtype,
                            void *stream);
 
+/* sma_attn_fwd_bool_mask that also leaves the mask's tile map behind.
+ *
+ *   map_out         NULL, or uint32 [Bm,Hm,T,2,TW] (contiguous; sma_tile_map_words(N) words per
+ *                   (batch entry, head) of the mask): receives exactly what sma_tile_map would
+ *                   write for packed_out, as a by-product of the same launch, for callers who go
+ *                   on to sma_attn_bwd_map (or to sma_attn_fwd_map with the same mask)
+ *
+ * Everything else as in sma_attn_fwd_bool_mask, which is this call with map_out = NULL.
+ *
+ * Replaces: as sma_attn_fwd_bool_mask; the map itself has no counterpart in the reference (its
+ *           kernel tests each 16 x 64 block after loading it, csrc/sparse_attention.cu:238-252).
+ */
+int sma_attn_fwd_bool_mask_map(const void *q, const void *k, const void *v, const uint8_t *mask,
+                               int64_t mask_stride_b, int64_t mask_stride_h, void *out, float *lse,
+                               uint32_t *packed_out, uint32_t *map_out, int B, int H, int N, int D,
+                               float scale, int dtype, void *stream);
+
 /* sma_attn_bwd for strided dout, q, k, v, out, dq, dk, dv and a shared mask (see
  * sma_attn_fwd_strided); lse and delta_ws are contiguous float [B,H,N].
  */

@@ -35,10 +35,9 @@
 //                 first kept score lies below the window.  The row maximum of a tile is not even
 //                 computed unless a row meets its first kept key there or the sum of the tile's
 //                 weights shows, afterwards, that a score has run away (then they are redone).
-//   skipping    = with a tile map (one "some bit set" and one "all bits set" bit per 128 x 64 block
-//                 of the mask, made by the packer) the work-group visits only the key tiles that
-//                 hold a set bit for its rows: no copies, no barrier for the others; a block whose
-//                 bits are all set needs no mask words and no bias.  Without a map every tile is
+//   skipping    = with a tile map (one "some bit set" bit per 64 x 64 block of the mask, made by
+//                 the packer) the work-group visits only the key tiles that hold a set bit for its
+//                 rows: no copies, no barrier for the others.  Without a map every tile is
 //                 copied.  Either way a wavefront whose own 32 x 64 block of mask bits is empty
 //                 skips its GEMMs and its softmax for that tile.
 //   head dim    = the description above is for 64.  128 runs the same code on two column halves of
@@ -91,7 +90,12 @@ template <int NH, bool BYTEMASK> struct Cfg {
     static constexpr int BYTE_SLOTS = NH == 1 ? 2 : 1;
     static constexpr int MASK_SLOT = BYTEMASK ? (BYTE_SLOTS - 1) * 8192 : 1024;     // distance between the slots
     static constexpr int OFF_LUT = OFF_MASK + (BYTEMASK ? BYTE_SLOTS * 8192 : NSTAGE * 1024);   // 16 x 16 B
-    static constexpr int LDS_BYTES = OFF_LUT + 256;
+    // byte mask only: the tile-map bits the wavefronts collect, [4 waves][MAP_WORDS][some, hole],
+    // and one arrival counter per pair of wavefronts (block of 64 rows)
+    static constexpr int MAP_WORDS = 32;                            // 32 x 32 key tiles: N <= 65536
+    static constexpr int OFF_MAP = OFF_LUT + 256;
+    static constexpr int OFF_MAP_ARRIVED = OFF_MAP + 4 * MAP_WORDS * 8;
+    static constexpr int LDS_BYTES = BYTEMASK ? OFF_MAP_ARRIVED + 16 : OFF_MAP;
 };
 
 template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_waitcnt vmcnt(%0)" :: "n"(N) : "memory"); }
@@ -99,7 +103,10 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_
 // PACKED_ROWS: the rows of q, k, v and out follow each other without gaps (row stride 64), as in
 // contiguous tensors; the strides between heads and batch entries stay free.  A row stride known
 // at compile time measured 0.25 us less fixed cost per launch than the same value read at run time.
-template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int HDIM, bool BYTEMASK = false>
+// BYPRODUCTS (with BYTEMASK): the caller wants the packed words and / or the tile map of the mask
+// left behind; a separate instantiation, so that the kernel of a caller who wants neither carries
+// none of that code (it measured 1.5 % on the headline workload even when switched off at run time).
+template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int HDIM, bool BYTEMASK = false, bool BYPRODUCTS = false>
 __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel(const AttnArgs a)
 {
     using E = Elem<BF16>;
@@ -216,13 +223,26 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     // like the mask; a mask shared between batch entries / heads is written by the first of them)
     const int qrow = qt * BM + wave * 32 + l32;
     uint32_t *words_out = nullptr;
-    if constexpr (BYTEMASK) {
+    // ... and where the tile map of this work-group's two blocks of 64 rows goes ([Bm, Hm, T, 2, TW]).
+    // Each wavefront notes per key tile whether its 32 rows hold a set bit and whether they hold a
+    // clear one, 32 tiles to a pair of registers that goes to LDS when it is full.  After
+    // its last tile a wavefront counts itself in; the second of a block's two to do so combines
+    // both and writes the block's words, which then travel while the output is being stored.
+    // (Per-lane bits ORed into LDS by all lanes at once, instead of the two ballots per tile,
+    // measured 4 us slower on the headline workload: 64 atomics on one address.)
+    uint32_t *map_dst = nullptr;
+    uint32_t some_acc = 0u, hole_acc = 0u;
+    u32x4 pend = {0u, 0u, 0u, 0u};        // packed words waiting to be stored, see mask_words
+    if constexpr (BYPRODUCTS) {
         const bool writer = (a.mask.sb != 0 || bi == 0) && (a.mask.sh != 0 || hi == 0);
-        if (a.mask_out != nullptr && writer) {
-            const int Hm = a.mask.sh != 0 ? a.H : 1;
-            const size_t slab_m = (size_t)((a.mask.sb != 0 ? bi : 0) * Hm + (a.mask.sh != 0 ? hi : 0));
-            words_out = a.mask_out + (slab_m * N + (qrow < N ? qrow : 0)) * nw;
-        }
+        const int Hm = a.mask.sh != 0 ? a.H : 1;
+        const size_t slab_m = (size_t)((a.mask.sb != 0 ? bi : 0) * Hm + (a.mask.sh != 0 ? hi : 0));
+        if (a.mask_out != nullptr && writer) words_out = a.mask_out + (slab_m * N + (qrow < N ? qrow : 0)) * nw;
+        if (a.map_out != nullptr && writer) map_dst = a.map_out + (slab_m * T + 2 * qt) * 2 * TW;
+    }
+    const uint32_t map_lds = lds0 + C::OFF_MAP + wave * (C::MAP_WORDS * 8);
+    if constexpr (BYPRODUCTS) {     // ordered before any arrival by the barriers of the main loop (T >= 1)
+        if (tid < 2) *(LDS_PTR(uint32_t))(uintptr_t)(lds0 + C::OFF_MAP_ARRIVED + 4 * tid) = 0u;
     }
     const uint32_t maddr = BYTEMASK ? lds0 + OFF_MASK + wave * 2048 + l32 * 64 : lds0 + OFF_MASK + wave * 256 + l32 * 8;
     const int msw = (l32 >> 2) & 3;
@@ -253,12 +273,52 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
                 const uint32_t hi = (mine >> 16) >> (part == 2 * hh + 1 ? shift : 0);
                 mine = (lo | (hi << 16)) & (hh ? a.last_mask1 : a.last_mask0);       // bits of keys >= N
             }
-            // a caller who will need the packed words (for the backward) gets them as a by-product
-            if (words_out != nullptr && qrow < N && 2 * x + hh < nw) words_out[2 * x + hh] = mine;
+            if (BYPRODUCTS && map_dst != nullptr) {
+                // rows beyond N repeat row N - 1 and change nothing; key bits beyond N are not valid
+                const uint32_t valid = x == T - 1 ? (hh ? a.last_mask1 : a.last_mask0) : 0xffffffffu;
+                const uint32_t some = __builtin_amdgcn_ballot_w64(mine != 0u) != 0ull ? 1u : 0u;
+                const uint32_t hole = __builtin_amdgcn_ballot_w64(mine != valid) != 0ull ? 1u : 0u;
+                some_acc |= some << (x & 31);
+                hole_acc |= hole << (x & 31);
+                if ((x & 31) == 31 || x == T - 1) {
+                    if (lane == 0) *(LDS_PTR(u32x2))(uintptr_t)(map_lds + (uint32_t)(x >> 5) * 8) = u32x2{some_acc, hole_acc};
+                    some_acc = hole_acc = 0u;
+                }
+            }
             // lanes < 32 hold the word of keys 0..31, lanes >= 32 that of keys 32..63: both to both
             const auto r = __builtin_amdgcn_permlane32_swap(mine, mine, false, false);
             w.x = (uint32_t)r[0];
             w.y = (uint32_t)r[1];
+            // A caller who will need the packed words (for the backward) gets them as a by-product.
+            // Stored tile by tile they would leave as 4-byte pieces of 64 different rows; instead
+            // the lower lane half keeps the words of tiles 4g and 4g + 1, the upper half those of
+            // tiles 4g + 2 and 4g + 3, and after every fourth tile each lane stores 16 bytes: 32
+            // consecutive bytes of each row per store instruction.
+            if (BYPRODUCTS && words_out != nullptr) {
+                const int j = x & 3;
+                const bool turn = hh == (j >> 1);
+                if ((j & 1) == 0) {
+                    pend.x = turn ? w.x : pend.x;
+                    pend.y = turn ? w.y : pend.y;
+                } else {
+                    pend.z = turn ? w.x : pend.z;
+                    pend.w = turn ? w.y : pend.w;
+                }
+                if (j == 3 || x == T - 1) {
+                    // words of tiles beyond the last one have indices >= nw and stay unwritten
+                    const int wb = 8 * (x >> 2) + 4 * hh;
+                    if (qrow < N) {
+                        typedef uint32_t u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+                        if (wb + 3 < nw) {
+                            __builtin_nontemporal_store((u32x4_a4)pend, reinterpret_cast<u32x4_a4 *>(words_out + wb));
+                        } else {
+                            if (wb < nw) words_out[wb] = pend.x;
+                            if (wb + 1 < nw) words_out[wb + 1] = pend.y;
+                            if (wb + 2 < nw) words_out[wb + 2] = pend.z;
+                        }
+                    }
+                }
+            }
         } else {
             w = lds_read_b64(maddr + slot * MASK_SLOT);
             const bool last = (x == T - 1);
@@ -610,6 +670,26 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     }
     wait_vmcnt<0>();              // no copy may outlive the work-group's LDS allocation
 
+    if constexpr (BYPRODUCTS) {
+        if (map_dst != nullptr) {
+            const int rb = wave >> 1;                          // block of 64 rows
+            uint32_t before = 0u;
+            if (lane == 0)
+                before = __hip_atomic_fetch_add((LDS_PTR(uint32_t))(uintptr_t)(lds0 + C::OFF_MAP_ARRIVED + 4 * rb), 1u,
+                                                __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_WORKGROUP);
+            before = __builtin_amdgcn_readfirstlane(before);
+            if (before == 1u && lane < TW && 2 * qt + rb < T) {
+                const int w = lane;                            // word of 32 key tiles
+                const uint32_t src = lds0 + C::OFF_MAP + (uint32_t)(2 * rb) * (C::MAP_WORDS * 8) + (uint32_t)w * 8;
+                const u32x2 x0 = lds_read_b64(src), x1 = lds_read_b64(src + C::MAP_WORDS * 8);
+                const uint32_t in_range = (w == TW - 1 && (T & 31)) ? ((1u << (T & 31)) - 1u) : 0xffffffffu;
+                uint32_t *dst = map_dst + (size_t)rb * 2 * TW;
+                dst[w] = (x0.x | x1.x) & in_range;
+                dst[TW + w] = ~(x0.y | x1.y) & in_range;
+            }
+        }
+    }
+
     // ---- epilogue ----
     // out = O / l.  The accumulator layout gives a lane 8-byte pieces of one row; written as they
     // are, a store instruction would touch 32 different 128-byte rows.  Each wave therefore
@@ -688,12 +768,17 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     default: kernel = attn_fwd_kernel<true, true, true, HDIM>; break;                  \
     }
 #define SMA_FWD_BYTEMASK_VARIANTS(HDIM)                                                 \
-    switch (variant >> 1) {                                                            \
+    switch ((variant >> 1) | (byproducts ? 4 : 0)) {                                   \
     case 0: kernel = attn_fwd_kernel<false, false, true, HDIM, true>; break;           \
     case 1: kernel = attn_fwd_kernel<false, true, true, HDIM, true>; break;            \
     case 2: kernel = attn_fwd_kernel<true, false, true, HDIM, true>; break;            \
-    default: kernel = attn_fwd_kernel<true, true, true, HDIM, true>; break;            \
+    case 3: kernel = attn_fwd_kernel<true, true, true, HDIM, true>; break;             \
+    case 4: kernel = attn_fwd_kernel<false, false, true, HDIM, true, true>; break;     \
+    case 5: kernel = attn_fwd_kernel<false, true, true, HDIM, true, true>; break;      \
+    case 6: kernel = attn_fwd_kernel<true, false, true, HDIM, true, true>; break;      \
+    default: kernel = attn_fwd_kernel<true, true, true, HDIM, true, true>; break;      \
     }
+    const bool byproducts = a.mask_out != nullptr || a.map_out != nullptr;
     if (a.byte_mask) {
         // built for contiguous rows only (checked by the C-ABI layer)
         if (!packed || a.N < 16) return hipErrorInvalidValue;

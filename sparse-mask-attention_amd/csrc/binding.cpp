@@ -11,10 +11,11 @@
 //       `forward` as tile_map, key tiles without a set bit are neither loaded nor computed)
 //   backward(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, scale, tile_map=None) -> None   (called by the
 //       reference's Python API, python/sparse_attention.py:91-94, but absent from its binding)
-//   forward_bool_mask(q, k, v, mask, out, lse, scale, is_training, packed_out=None) -> None   (not in
+//   forward_bool_mask(q, k, v, mask, out, lse, scale, is_training, packed_out=None, map_out=None) -> None   (not in
 //       the reference: `forward` with the boolean mask itself in place of the packed one, one launch
 //       instead of pack_mask + forward; `packed_out`, if given, receives what pack_mask would
-//       return; `bool_mask_supported(q, k, v, mask)` says whether it applies)
+//       return and `map_out` what tile_map would return for it; `bool_mask_supported(q, k, v, mask)`
+//       says whether it applies)
 //
 // Differences, all on the safe side: `lse` may be None (the reference's own inference wrapper
 // passes None, python/sparse_attention.py:170-171); every tensor argument is checked (device,
@@ -145,7 +146,8 @@ bool bool_mask_supported(const torch::Tensor &q, const torch::Tensor &k, const t
 void forward_bool_mask(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,
                        const torch::Tensor &mask, torch::Tensor out,
                        const c10::optional<torch::Tensor> &lse, double scale, bool is_training,
-                       const c10::optional<torch::Tensor> &packed_out)
+                       const c10::optional<torch::Tensor> &packed_out,
+                       const c10::optional<torch::Tensor> &map_out)
 {
     TORCH_CHECK(q.is_cuda(), "q must be a GPU tensor");
     TORCH_CHECK(q.dim() == 4, "q must be 4D [B, H, N, D]");
@@ -179,16 +181,27 @@ void forward_bool_mask(const torch::Tensor &q, const torch::Tensor &k, const tor
                     "packed_out must be a contiguous int32 [mask.size(0), mask.size(1), N, ceil(N/32)] tensor on q's device");
         packed_ptr = reinterpret_cast<uint32_t *>(p.data_ptr<int32_t>());
     }
+    uint32_t *map_ptr = nullptr;
+    if (map_out.has_value() && map_out->defined()) {
+        const torch::Tensor &m = *map_out;
+        const int64_t T = (N + 63) / 64;
+        TORCH_CHECK(m.device() == q.device() && m.scalar_type() == at::kInt && m.dim() == 5 &&
+                        m.size(0) == mask.size(0) && m.size(1) == mask.size(1) && m.size(2) == T &&
+                        m.size(3) == 2 && m.size(4) == (T + 31) / 32 && m.is_contiguous(),
+                    "map_out must be a contiguous int32 [mask.size(0), mask.size(1), T, 2, ceil(T/32)] tensor "
+                    "on q's device, T = ceil(N/64)");
+        map_ptr = reinterpret_cast<uint32_t *>(m.data_ptr<int32_t>());
+    }
     const int64_t msb = mask.size(0) == 1 ? 0 : mask.size(1) * N * N;
     const int64_t msh = mask.size(1) == 1 ? 0 : N * N;
     const c10::DeviceGuard guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
-    const int st = sma_attn_fwd_bool_mask(q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                          reinterpret_cast<const uint8_t *>(mask.data_ptr<bool>()), msb, msh,
-                                          out.data_ptr(), lse_ptr, packed_ptr, (int)B, (int)H, (int)N, (int)D,
-                                          (float)scale, dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16,
-                                          stream);
-    check_status(st, "sma_attn_fwd_bool_mask");
+    const int st = sma_attn_fwd_bool_mask_map(q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                              reinterpret_cast<const uint8_t *>(mask.data_ptr<bool>()), msb, msh,
+                                              out.data_ptr(), lse_ptr, packed_ptr, map_ptr, (int)B, (int)H, (int)N,
+                                              (int)D, (float)scale,
+                                              dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
+    check_status(st, "sma_attn_fwd_bool_mask_map");
 }
 
 // backward(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, scale) -> None, the call the
@@ -293,7 +306,8 @@ PYBIND11_MODULE(sparse_attn_cuda, m)
     m.def("forward_bool_mask", &forward_bool_mask,
           "Sparse-mask attention forward straight from the bool mask (one launch; see bool_mask_supported)",
           py::arg("q"), py::arg("k"), py::arg("v"), py::arg("mask"), py::arg("out"), py::arg("lse"),
-          py::arg("scale"), py::arg("is_training"), py::arg("packed_out") = py::none());
+          py::arg("scale"), py::arg("is_training"), py::arg("packed_out") = py::none(),
+          py::arg("map_out") = py::none());
     m.def("bool_mask_supported", &bool_mask_supported,
           "Whether forward_bool_mask applies to these tensors (else use pack_mask + forward)", py::arg("q"),
           py::arg("k"), py::arg("v"), py::arg("mask"));

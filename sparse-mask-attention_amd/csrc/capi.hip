@@ -254,6 +254,7 @@ int sma_attn_fwd_map_strided(const sma_tensor *q, const sma_tensor *k, const sma
     a.D = D;
     a.byte_mask = 0;
     a.mask_out = nullptr;
+    a.map_out = nullptr;
     // the map is contiguous [Bm, Hm, ...] with the mask's own Bm, Hm (1 where the mask is shared)
     a.tile_map = tile_map;
     const long long map_words = sma_tile_map_words(N);
@@ -291,6 +292,15 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
                            uint32_t *packed_out, int B, int H, int N, int D, float scale, int dtype,
                            void *stream)
 {
+    return sma_attn_fwd_bool_mask_map(q, k, v, mask, mask_stride_b, mask_stride_h, out, lse, packed_out, nullptr, B,
+                                      H, N, D, scale, dtype, stream);
+}
+
+int sma_attn_fwd_bool_mask_map(const void *q, const void *k, const void *v, const uint8_t *mask,
+                               int64_t mask_stride_b, int64_t mask_stride_h, void *out, float *lse,
+                               uint32_t *packed_out, uint32_t *map_out, int B, int H, int N, int D,
+                               float scale, int dtype, void *stream)
+{
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
     if (D != 32 && D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
     if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
@@ -303,7 +313,7 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
     if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
     // a lane's byte offset into the mask of one (b,h) is a 32-bit register
     if ((long long)N * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
-    if ((lse && misaligned(lse, 4)) || (packed_out && misaligned(packed_out, 4)))
+    if ((lse && misaligned(lse, 4)) || (packed_out && misaligned(packed_out, 4)) || (map_out && misaligned(map_out, 4)))
         return SMA_ERR_ALIGNMENT;
     if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 
@@ -322,6 +332,7 @@ int sma_attn_fwd_bool_mask(const void *q, const void *k, const void *v, const ui
     a.D = D;
     a.byte_mask = 1;
     a.mask_out = packed_out;
+    a.map_out = map_out;
     a.tile_map = nullptr;
     a.map_sb = a.map_sh = 0;
     a.qtiles = (int)qtiles;

@@ -53,6 +53,7 @@ struct AttnArgs {
     int D;                          // head dim: 32, 64 or 128
     int byte_mask;                  // the mask is the caller's boolean tensor, not packed words
     uint32_t *mask_out;             // byte_mask only: nullptr, or where to leave the packed words [Bm, Hm, N, nw]
+    uint32_t *map_out;              // byte_mask only: nullptr, or where to leave the tile map (layout as tile_map below)
     // packed mask only: nullptr, or the tile map [Bm, Hm, T, 2, ceil(T/32)] (T = ceil(N/64)): per block
     // of 64 query rows one bit per 64-key tile "some mask bit set", then one bit per key tile "all
     // mask bits set"; strides between batch entries / heads in words, 0 = shared

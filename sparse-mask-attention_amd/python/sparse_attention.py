@@ -110,8 +110,8 @@ class SparseAttentionFunction(Function):
     """forward = fused HIP kernel (saves LSE); backward = the HIP dQ and dK/dV kernels.
 
     ``mask_packed`` may be None: the mask is then read as it is by the one-launch forward, which
-    leaves the packed words the backward needs as a by-product, or packed first where that kernel
-    does not apply."""
+    leaves the packed words and the tile map the backward uses as by-products, or packed first
+    where that kernel does not apply."""
 
     @staticmethod
     def forward(ctx, q, k, v, mask_packed, mask_bool, scale, seq_len, tile_map=None):
@@ -125,9 +125,15 @@ class SparseAttentionFunction(Function):
             if sparse_attn_cuda.bool_mask_supported(q, k, v, mask_bool):
                 mask_packed = torch.empty(mask_bool.shape[0], mask_bool.shape[1], N, (N + 31) // 32,
                                           device=q.device, dtype=torch.int32)
-                sparse_attn_cuda.forward_bool_mask(q, k, v, mask_bool, out, lse, scale, True, mask_packed)
+                # the same launch leaves the mask's tile map behind: the backward visits only the
+                # blocks that hold something
+                T = (N + 63) // 64
+                tile_map = torch.empty(mask_bool.shape[0], mask_bool.shape[1], T, 2, (T + 31) // 32,
+                                       device=q.device, dtype=torch.int32)
+                sparse_attn_cuda.forward_bool_mask(q, k, v, mask_bool, out, lse, scale, True, mask_packed, tile_map)
                 ctx.save_for_backward(q, k, v, out, lse, mask_packed)
                 ctx.scale = scale
+                ctx.tile_map = tile_map
                 return out
             mask_packed = pack_mask(mask_bool)
         sparse_attn_cuda.forward(q, k, v, mask_packed, out, lse, scale, True, tile_map)

@@ -77,6 +77,8 @@ def load():
         lib.sma_attn_bwd_map_strided.argtypes = [tp] * 5 + [vp, vp, i64, i64, vp, tp, tp, tp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_fwd_bool_mask.restype = ci
         lib.sma_attn_fwd_bool_mask.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_attn_fwd_bool_mask_map.restype = ci
+        lib.sma_attn_fwd_bool_mask_map.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         _lib = lib
     return _lib
 
@@ -274,10 +276,12 @@ def attn_bwd_strided(dout, q, k, v, out, lse, packed, grads=None, scale=None):
     return dq, dk, dv, delta
 
 
-def attn_fwd_bool_mask(q, k, v, mask, scale=None, want_lse=False, expect=SMA_OK, want_packed=False):
+def attn_fwd_bool_mask(q, k, v, mask, scale=None, want_lse=False, expect=SMA_OK, want_packed=False,
+                       want_map=False):
     """Forward straight from the boolean mask ([1|B, 1|H, N, N], contiguous) through
-    sma_attn_fwd_bool_mask; returns out (and lse) (and the packed words it leaves behind), or the
-    status if `expect` is an error code."""
+    sma_attn_fwd_bool_mask (sma_attn_fwd_bool_mask_map with `want_map`); returns out (and lse) (and
+    the packed words it leaves behind) (and the tile map), or the status if `expect` is an error
+    code."""
     lib = load()
     B, H, N, D = q.shape
     if scale is None:
@@ -291,11 +295,18 @@ def attn_fwd_bool_mask(q, k, v, mask, scale=None, want_lse=False, expect=SMA_OK,
     lse = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device) if want_lse else None
     packed = (torch.full((Bm, Hm, N, (N + 31) // 32), -1431655766, dtype=torch.int32, device=q.device)
               if want_packed else None)
-    st = lib.sma_attn_fwd_bool_mask(q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), msb, msh,
-                                    out.data_ptr(), lse.data_ptr() if want_lse else None,
-                                    packed.data_ptr() if want_packed else None, B, H, N, D, scale, dt, _stream())
+    if want_map:
+        tm = _new_map(Bm, Hm, N, q.device)
+        st = lib.sma_attn_fwd_bool_mask_map(q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), msb, msh,
+                                            out.data_ptr(), lse.data_ptr() if want_lse else None,
+                                            packed.data_ptr() if want_packed else None, tm.data_ptr(), B, H, N, D,
+                                            scale, dt, _stream())
+    else:
+        st = lib.sma_attn_fwd_bool_mask(q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), msb, msh,
+                                        out.data_ptr(), lse.data_ptr() if want_lse else None,
+                                        packed.data_ptr() if want_packed else None, B, H, N, D, scale, dt, _stream())
     if expect != SMA_OK:
         return st
     assert st == SMA_OK, lib.sma_strerror(st)
-    res = (out,) + ((lse,) if want_lse else ()) + ((packed,) if want_packed else ())
+    res = (out,) + ((lse,) if want_lse else ()) + ((packed,) if want_packed else ()) + ((tm,) if want_map else ())
     return res if len(res) > 1 else out

@@ -378,6 +378,28 @@ def test_inference_entry_point_reads_the_bool_mask_itself(sa, dev, monkeypatch):
     assert torch.allclose(o32.cpu(), ref, atol=1e-2, rtol=2e-2)
 
 
+def test_autograd_from_a_bool_mask_with_empty_blocks_uses_the_map_and_changes_nothing(sa, dev):
+    """With a bool mask the one-launch forward hands the backward the packed words and the tile map;
+    the gradients are those of the path that packs first and walks every tile, bit for bit."""
+    g = torch.Generator().manual_seed(21)
+    B, H, N = 2, 3, 320
+    blocks = torch.rand(B, H, 5, 5, generator=g) < 0.3
+    mask = (blocks.repeat_interleave(64, 2).repeat_interleave(64, 3) & (torch.rand(B, H, N, N, generator=g) < 0.5))
+    q, k, v, do = (torch.randn(B, H, N, 64, generator=g).half().to(dev) for _ in range(4))
+    md = mask.to(dev)
+    grads = []
+    for kw in ({}, {"mask_packed": sa.pack_mask(md)}):
+        leaves = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        out = sa.sparse_attention(*leaves, None if kw else md, **kw)
+        out.backward(do)
+        grads.append([out.detach()] + [t.grad for t in leaves])
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
+    wanted = O.sparse_attention_bwd_ref(q.float().cpu(), k.float().cpu(), v.float().cpu(), mask, do.float().cpu())
+    for got, want in zip(grads[0][1:], wanted):
+        assert torch.allclose(got.float().cpu(), want, atol=1e-4 + 1e-2 * want.abs().max().item(), rtol=1e-2)
+
+
 def test_mfma_stream_probe_runs_and_reports_a_clock(dev):
     """The benchmark's yardstick kernel: finishes, and the two tick counts it leaves give a shader
     clock that a GPU of this kind can have."""

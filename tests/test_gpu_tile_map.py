@@ -1,4 +1,5 @@
-"""GPU parity of the tile map (sma_tile_map, sma_pack_mask_map) against the oracle, bit for bit, and
+"""GPU parity of the tile map (sma_tile_map, sma_pack_mask_map, and the one the forward from the
+boolean mask leaves behind, sma_attn_fwd_bool_mask_map) against the oracle, bit for bit, and
 of the forward that walks it (sma_attn_fwd_map): the same output and lse, bit for bit, as the forward
 that visits every tile, on masks with empty blocks, empty block rows, full blocks and ragged
 edges, at all head dims and both dtypes, and on the benchmark workloads at full size."""
@@ -53,6 +54,56 @@ def test_tile_map_matches_the_oracle(dev, N):
             dirty = packed.clone()
             dirty[..., -1] |= -(1 << (N % 32))
             assert np.array_equal(_capi.tile_map(dirty).cpu().numpy(), want), (name, N, "dirty pad bits")
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("N", [16, 17, 63, 64, 65, 127, 128, 129, 200, 256, 333, 512, 1000])
+def test_forward_from_bool_mask_leaves_the_tile_map(dev, N, D, dtype):
+    """The map that comes out of the one-launch forward equals the oracle's, with and without the
+    packed words being asked for, and asking for it changes neither the output nor the lse."""
+    g = torch.Generator().manual_seed(31 * N + D)
+    q, k, v = (torch.randn(2, 2, N, D, generator=g).to(dtype).to(dev) for _ in range(3))
+    for name, mask in _masks(N, g):
+        B = mask.shape[0]
+        qq, kk, vv = q[:B], k[:B], v[:B]
+        m = mask.to(dev)
+        want_out, want_lse = _capi.attn_fwd_bool_mask(qq, kk, vv, m, want_lse=True)
+        out, lse, packed, tm = _capi.attn_fwd_bool_mask(qq, kk, vv, m, want_lse=True, want_packed=True, want_map=True)
+        out2, tm2 = _capi.attn_fwd_bool_mask(qq, kk, vv, m, want_map=True)
+        torch.cuda.synchronize()
+        want = O.tile_map_ref(mask).view(np.int32)
+        assert np.array_equal(tm.cpu().numpy(), want), (name, N, D, dtype)
+        assert np.array_equal(tm2.cpu().numpy(), want), (name, N, D, dtype, "map only")
+        assert np.array_equal(packed.cpu().numpy(), O.pack_mask_ref(mask)), (name, N, D, dtype)
+        assert torch.equal(out, want_out) and torch.equal(lse, want_lse) and torch.equal(out2, want_out), (name, N, D)
+
+
+def test_bool_mask_tile_map_of_a_shared_mask_and_of_odd_bytes(dev):
+    g = torch.Generator().manual_seed(5)
+    B, H, N = 3, 4, 300
+    q, k, v = (torch.randn(B, H, N, 64, generator=g).half().to(dev) for _ in range(3))
+    for shape in [(1, 1), (B, 1), (1, H), (B, H)]:
+        mask = _block_mask(shape[0], shape[1], N, g, keep=0.3, inner=0.6)
+        # bytes other than 0 and 1 count as set
+        raw = mask.to(torch.uint8) * torch.randint(1, 256, mask.shape, generator=g, dtype=torch.int32).to(torch.uint8)
+        out, packed, tm = _capi.attn_fwd_bool_mask(q, k, v, raw.to(dev).view(torch.bool), want_packed=True, want_map=True)
+        torch.cuda.synchronize()
+        assert np.array_equal(tm.cpu().numpy(), O.tile_map_ref(mask).view(np.int32)), shape
+        assert np.array_equal(packed.cpu().numpy(), O.pack_mask_ref(mask)), shape
+        assert torch.equal(_capi.tile_map(packed), tm), shape
+
+
+def test_bool_mask_tile_map_with_more_than_32_key_tiles(dev):
+    N = 64 * 33 + 5
+    g = torch.Generator().manual_seed(11)
+    mask = torch.rand(1, 2, N, N, generator=g) < 0.0005
+    mask[0, 0, :64, 64 * 32: 64 * 33] = True
+    mask[0, 1, 64 * 32:, :] = True                                    # full blocks up to the ragged corner
+    q, k, v = (torch.randn(1, 2, N, 64, generator=g).half().to(dev) for _ in range(3))
+    out, tm = _capi.attn_fwd_bool_mask(q, k, v, mask.to(dev), want_map=True)
+    torch.cuda.synchronize()
+    assert np.array_equal(tm.cpu().numpy(), O.tile_map_ref(mask).view(np.int32))
 
 
 def test_tile_map_with_more_than_32_key_tiles(dev):
