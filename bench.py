@@ -91,20 +91,48 @@ def cpu_model():
     return "unknown"
 
 
+# The source files each profiled kernel is compiled from: a counter summary under profiles/ records
+# their digest, so that a figure recorded for other code than the one that runs now is not passed on.
+KERNEL_SOURCES = {
+    "attn_fwd_kernel": ("attn_fwd.hip", "attn_common.h", "sma_internal.h"),
+    "attn_fwd_bool_mask_kernel": ("attn_fwd.hip", "attn_common.h", "sma_internal.h"),
+    "pack_mask_kernel": ("pack_mask.hip", "sma_internal.h"),
+    "attn_bwd_dq_kernel": ("attn_bwd.hip", "attn_common.h", "sma_internal.h"),
+    "attn_bwd_dkv_kernel": ("attn_bwd.hip", "attn_common.h", "sma_internal.h"),
+}
+
+
+def source_digest(kernel):
+    """First 16 hex digits of the SHA-256 of the kernel's source files, in the order listed."""
+    import hashlib
+    h = hashlib.sha256()
+    for name in KERNEL_SOURCES[kernel]:
+        with open(os.path.join(ROOT, "sparse-mask-attention_amd", "csrc", name), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
 def measured_traffic(workload, *kernels):
     """HBM bytes per launch (summed over `kernels`) from the committed rocprofv3 counter summaries
     of this workload (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a
-    plain copy of known size); None when a summary for this workload is not there.  Counters cannot
-    be read from inside this process, so the figure is the recorded one, not a live one."""
+    plain copy of known size).  Counters cannot be read from inside this process, so the figure is
+    the recorded one, not a live one: None when a summary for this workload is not there, or when
+    it was recorded for other kernel sources than the ones in the tree now."""
     import re
     total = 0
     for kernel in kernels:
         path = os.path.join(ROOT, "profiles", f"{kernel}_{workload}.txt")
         try:
-            m = re.search(r"traffic per launch ([0-9.]+) MB", open(path).read())
+            text = open(path).read()
         except OSError:
             return None
-        if not m:
+        m = re.search(r"traffic per launch ([0-9.]+) MB", text)
+        d = re.search(r"sources sha256/16: ([0-9a-f]{16})", text)
+        try:
+            current = source_digest(kernel)
+        except OSError:
+            return None
+        if not m or not d or d.group(1) != current:
             return None
         total += int(float(m.group(1)) * 1e6)
     return total

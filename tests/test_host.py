@@ -178,3 +178,25 @@ def test_structured_masks():
     assert not torch.triu(m[0, 0], diagonal=1).any() and torch.diagonal(m[0, 0]).all()
     tf, pct = harness.compute_mfu(1.0, 16, 12, 512, 64, 2516.6)
     assert tf == pytest.approx(12.884901888) and pct == pytest.approx(100 * 12.884901888 / 2516.6)
+
+
+def test_bench_passes_on_recorded_traffic_only_for_the_sources_it_was_recorded_for(tmp_path, monkeypatch):
+    """bench.py cannot read HBM counters itself and quotes them from the summaries under profiles/;
+    a summary made for other kernel sources than those in the tree must not be quoted."""
+    sys.path.insert(0, ROOT)
+    import bench
+    csrc = tmp_path / "sparse-mask-attention_amd" / "csrc"
+    csrc.mkdir(parents=True)
+    for name in ("pack_mask.hip", "sma_internal.h"):
+        (csrc / name).write_text("// " + name + "\n")
+    monkeypatch.setattr(bench, "ROOT", str(tmp_path))
+    digest = bench.source_digest("pack_mask_kernel")
+    assert re.fullmatch(r"[0-9a-f]{16}", digest)
+    prof = tmp_path / "profiles"
+    prof.mkdir()
+    (prof / "pack_mask_kernel_C2.txt").write_text(
+        f"kernel sources (...), sources sha256/16: {digest}\n  traffic per launch 56.65 MB vs algorithmic 56.62 MB\n")
+    assert bench.measured_traffic("C2", "pack_mask_kernel") == 56650000
+    assert bench.measured_traffic("C3", "pack_mask_kernel") is None            # no summary
+    (csrc / "pack_mask.hip").write_text("// changed\n")
+    assert bench.measured_traffic("C2", "pack_mask_kernel") is None            # recorded for other code
