@@ -315,6 +315,9 @@ int sma_attn_fwd_bool_mask_map(const void *q, const void *k, const void *v, cons
     if ((long long)N * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
     if ((lse && misaligned(lse, 4)) || (packed_out && misaligned(packed_out, 4)) || (map_out && misaligned(map_out, 4)))
         return SMA_ERR_ALIGNMENT;
+    // the kernel collects the map in 32 words of 32 key tiles per wavefront (N <= 65536; the limit on
+    // N * N above is the tighter one)
+    if (map_out && (N + 63) / 64 > 32 * 32) return SMA_ERR_BAD_SHAPE;
     if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 
     sma::AttnArgs a;
