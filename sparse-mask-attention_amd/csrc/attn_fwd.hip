@@ -255,16 +255,32 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
             // a byte counts as "attend" when it is non-zero, as in the packer: nz() leaves 0x80 in
             // every non-zero byte, the dot products weigh those with 1, 2, 4 .. 128 (times 128)
             auto nz = [](uint32_t x) -> uint32_t { return (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u; };
-            uint32_t b0 = __builtin_amdgcn_udot4(nz(d0.x), 0x08040201u, 0u, false);
-            uint32_t b1 = __builtin_amdgcn_udot4(nz(d0.z), 0x08040201u, 0u, false);
-            uint32_t b2 = __builtin_amdgcn_udot4(nz(d1.x), 0x08040201u, 0u, false);
-            uint32_t b3 = __builtin_amdgcn_udot4(nz(d1.z), 0x08040201u, 0u, false);
-            b0 = __builtin_amdgcn_udot4(nz(d0.y), 0x80402010u, b0, false);
-            b1 = __builtin_amdgcn_udot4(nz(d0.w), 0x80402010u, b1, false);
-            b2 = __builtin_amdgcn_udot4(nz(d1.y), 0x80402010u, b2, false);
-            b3 = __builtin_amdgcn_udot4(nz(d1.w), 0x80402010u, b3, false);
-            // each partial value is 128 x (8 bits): bits 7..14
-            uint32_t mine = (b0 >> 7) | (b1 << 1) | (b2 << 9) | (b3 << 17);
+            // ... which costs three instructions per four bytes.  Bytes that are all 0 or 1 (every
+            // mask PyTorch itself made) need none of it: one look at the wavefront's 2 KiB decides.
+            const uint32_t other = (d0.x | d0.y | d0.z | d0.w | d1.x | d1.y | d1.z | d1.w) & 0xfefefefeu;
+            uint32_t mine;
+            if (__builtin_amdgcn_ballot_w64(other != 0u) == 0ull) {
+                uint32_t b0 = __builtin_amdgcn_udot4(d0.x, 0x08040201u, 0u, false);
+                uint32_t b1 = __builtin_amdgcn_udot4(d0.z, 0x08040201u, 0u, false);
+                uint32_t b2 = __builtin_amdgcn_udot4(d1.x, 0x08040201u, 0u, false);
+                uint32_t b3 = __builtin_amdgcn_udot4(d1.z, 0x08040201u, 0u, false);
+                b0 = __builtin_amdgcn_udot4(d0.y, 0x80402010u, b0, false);
+                b1 = __builtin_amdgcn_udot4(d0.w, 0x80402010u, b1, false);
+                b2 = __builtin_amdgcn_udot4(d1.y, 0x80402010u, b2, false);
+                b3 = __builtin_amdgcn_udot4(d1.w, 0x80402010u, b3, false);
+                mine = b0 | (b1 << 8) | (b2 << 16) | (b3 << 24);
+            } else {
+                uint32_t b0 = __builtin_amdgcn_udot4(nz(d0.x), 0x08040201u, 0u, false);
+                uint32_t b1 = __builtin_amdgcn_udot4(nz(d0.z), 0x08040201u, 0u, false);
+                uint32_t b2 = __builtin_amdgcn_udot4(nz(d1.x), 0x08040201u, 0u, false);
+                uint32_t b3 = __builtin_amdgcn_udot4(nz(d1.z), 0x08040201u, 0u, false);
+                b0 = __builtin_amdgcn_udot4(nz(d0.y), 0x80402010u, b0, false);
+                b1 = __builtin_amdgcn_udot4(nz(d0.w), 0x80402010u, b1, false);
+                b2 = __builtin_amdgcn_udot4(nz(d1.y), 0x80402010u, b2, false);
+                b3 = __builtin_amdgcn_udot4(nz(d1.w), 0x80402010u, b3, false);
+                // each partial value is 128 x (8 bits): bits 7..14
+                mine = (b0 >> 7) | (b1 << 1) | (b2 << 9) | (b3 << 17);
+            }
             if (x == T - 1) {
                 // the chunk that holds the row's end was copied from 16 bytes before that end: its
                 // bits move down to their places (zeros follow them)
