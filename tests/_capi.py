@@ -276,6 +276,25 @@ def attn_bwd_strided(dout, q, k, v, out, lse, packed, grads=None, scale=None):
     return dq, dk, dv, delta
 
 
+def attn_bwd_map_strided(dout, q, k, v, out, lse, packed, tm, scale=None):
+    """Backward through sma_attn_bwd_map_strided (any views, shared masks, tile map of `packed`);
+    returns new contiguous (dq, dk, dv)."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    dq, dk, dv = (torch.full((B, H, N, D), float("nan"), dtype=q.dtype, device=q.device) for _ in range(3))
+    delta = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device)
+    msb, msh = _mask_strides(packed, B, H)
+    ts = [SmaTensor.of(t) for t in (dout, q, k, v, out, dq, dk, dv)]
+    st = lib.sma_attn_bwd_map_strided(ts[0], ts[1], ts[2], ts[3], ts[4], lse.data_ptr(), packed.data_ptr(), msb, msh,
+                                      tm.data_ptr(), ts[5], ts[6], ts[7], delta.data_ptr(), B, H, N, D, scale, dt,
+                                      _stream())
+    assert st == SMA_OK, lib.sma_strerror(st)
+    return dq, dk, dv
+
+
 def attn_fwd_bool_mask(q, k, v, mask, scale=None, want_lse=False, expect=SMA_OK, want_packed=False,
                        want_map=False):
     """Forward straight from the boolean mask ([1|B, 1|H, N, N], contiguous) through

@@ -76,6 +76,23 @@ def test_random_configuration(dev, seed):
     dq, dk, dv, _ = _capi.attn_bwd_strided(dod, qd, kd, vd, out, lse, packed, grads=grads, scale=scale)
     torch.cuda.synchronize()
 
+    # the same through the tile map, and (where it applies) through the one launch that reads the
+    # boolean mask and leaves packed words and map behind: bit for bit what was computed above
+    tm = _capi.tile_map(packed)
+    assert torch.equal(tm.cpu(), torch.from_numpy(O.tile_map_ref(mask).view("int32"))), tag
+    out_m, lse_m = _capi.attn_fwd_map_strided(qd, kd, vd, packed, tm, scale=scale, want_lse=True)
+    assert torch.equal(out_m, out.contiguous()) and torch.equal(lse_m, lse), tag
+    got_m = _capi.attn_bwd_map_strided(dod, qd, kd, vd, out, lse, packed, tm, scale=scale)
+    for name, a, b_ in zip(("dq", "dk", "dv"), got_m, (dq, dk, dv)):
+        assert torch.equal(a, b_.contiguous()), f"{name} with map {tag}"
+    if N >= 16:
+        qc, kc, vc = (t.contiguous() for t in (qd, kd, vd))
+        out_b, lse_b, packed_b, tm_b = _capi.attn_fwd_bool_mask(qc, kc, vc, mask.to(dev), scale=scale, want_lse=True,
+                                                                want_packed=True, want_map=True)
+        assert torch.equal(packed_b, packed) and torch.equal(tm_b, tm), tag
+        assert torch.equal(out_b, out.contiguous()) and torch.equal(lse_b, lse), tag
+    torch.cuda.synchronize()
+
     full = mask.expand(B, H, N, N)
     sharp = max(1.0, abs(scale) * math.sqrt(D)) if scale is not None else 1.0
     ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), full, scale=scale)
