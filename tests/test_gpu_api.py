@@ -2,6 +2,7 @@
 same calls a user of the reference makes, checked against the oracle."""
 import importlib
 import math
+import os
 import sys
 
 import numpy as np
@@ -416,3 +417,20 @@ def test_mfma_stream_probe_runs_and_reports_a_clock(dev):
         assert 0.3 < ghz < 3.0, ghz
     assert lib.sma_probe_mfma_stream(1, 10, 0, None, None) == _capi.SMA_OK
     assert lib.sma_probe_mfma_stream(1, 10, 4, None, None) == _capi.SMA_ERR_NULL_POINTER
+
+
+def test_command_line_harness_acceptance_run_and_sweeps(dev, capsys):
+    """run.py: the reference's acceptance run (run.py:349-404 there) passes, and the sweep tables
+    print a row for every size with a latency above zero."""
+    import importlib
+    pkg = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "sparse-mask-attention_amd")
+    if pkg not in sys.path:
+        sys.path.insert(0, pkg)
+    run = importlib.import_module("run")
+    assert run.run_correctness(dev) is True
+    text = capsys.readouterr().out
+    assert text.count("[PASS]") == 5 and "FAIL" not in text
+    run.run_perf(dev)
+    rows = [line.split() for line in capsys.readouterr().out.splitlines() if line.strip()[:1].isdigit()]
+    assert [int(r[0]) for r in rows] == [64, 128, 256, 512, 1024, 1, 4, 8, 16, 32, 64]
+    assert all(float(r[1]) > 0 and float(r[2]) > 0 for r in rows)
