@@ -145,6 +145,14 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="C2", choices=["C1", "C2", "C3", "C4", "C5"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--only", default=None,
+                    choices=["packed", "packed_map", "fused", "fused_training", "pack", "bwd", "bwd_map"],
+                    help="launch ONE kind of kernel back to back (--warmup, then --steps launches), print its "
+                         "mean time and exit: packed = packed-mask forward over all tiles, packed_map = the same "
+                         "walking the mask's tile map, fused = forward from the boolean mask, fused_training = "
+                         "the same leaving lse, packed words and tile map behind, pack = the packer, bwd / "
+                         "bwd_map = the backward without / with the tile map.  For rocprofv3 runs whose "
+                         "per-kernel averages must not blend launch contexts.")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also run one plain device-to-device copy of this many MiB (a traffic yardstick "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
@@ -174,6 +182,29 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
+
+    if args.only:
+        packed = ext.pack_mask(md)
+        out = torch.empty_like(qd)
+        full_map = ext.tile_map(packed)         # the map itself, whether or not walking it pays
+        lse = torch.empty(w.B, w.H, w.N, dtype=torch.float32, device=dev)
+        if args.only in ("bwd", "bwd_map"):
+            ext.forward(qd, kd, vd, packed, out, lse, scale, True)
+            dout = torch.randn(qd.shape, generator=torch.Generator().manual_seed(43)).to(qd.dtype).to(dev)
+            dq, dk, dv = (torch.empty_like(qd) for _ in range(3))
+        packed2, map2 = torch.empty_like(packed), torch.empty_like(full_map)
+        fn = {
+            "packed": lambda: ext.forward(qd, kd, vd, packed, out, None, scale, False),
+            "packed_map": lambda: ext.forward(qd, kd, vd, packed, out, None, scale, False, full_map),
+            "fused": lambda: ext.forward_bool_mask(qd, kd, vd, md, out, None, scale, False),
+            "fused_training": lambda: ext.forward_bool_mask(qd, kd, vd, md, out, lse, scale, True, packed2, map2),
+            "pack": lambda: ext.pack_mask(md),
+            "bwd": lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale),
+            "bwd_map": lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale, full_map),
+        }[args.only]
+        ms = event_time_ms(fn, args.warmup, args.steps, torch)
+        print(json.dumps({"only": args.only, "workload": w.name, "launches": args.steps, "ms": round(ms, 5)}), flush=True)
+        return
 
     def step_two_launches():
         packed = ext.pack_mask(md)
@@ -344,14 +375,16 @@ def main():
         result["roofline"] = dict(result["roofline_attn"])
 
     # ---- what this GPU sustains on a pure stream of the kernels' MFMA, and at what clock ----
-    lib.sma_probe_mfma_stream.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    # (benchmark infrastructure in a library of its own, benchprobe/mfma_probe.h: not part of libsma_hip.so)
+    probe_lib = ctypes.CDLL(os.path.join(PKG, "libsma_probe.so"))
+    probe_lib.sma_probe_mfma_stream.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
     n_cu = torch.cuda.get_device_properties(0).multi_processor_count
     stamps = torch.zeros(2 * n_cu, dtype=torch.int64, device=dev)
     probe = {}
     for label, rnd in (("zero_operands", 0), ("random_operands", 1)):
         iters = 20000
-        lib.sma_probe_mfma_stream(rnd, 2000, n_cu, stamps.data_ptr(), stream)
-        ms = event_time_ms(lambda: lib.sma_probe_mfma_stream(rnd, iters, n_cu, stamps.data_ptr(), stream), 1, 3, torch)
+        probe_lib.sma_probe_mfma_stream(rnd, 2000, n_cu, stamps.data_ptr(), stream)
+        ms = event_time_ms(lambda: probe_lib.sma_probe_mfma_stream(rnd, iters, n_cu, stamps.data_ptr(), stream), 1, 3, torch)
         st = stamps.view(n_cu, 2).double().cpu()
         flops = n_cu * 12 * 8 * iters * 2.0 * 32 * 32 * 16
         probe[label] = {"tflops": round(flops / (ms * 1e-3) / 1e12, 1),

@@ -4,7 +4,9 @@
  * the GPU that is current on the calling thread; `stream` is a hipStream_t passed as void*
  * (NULL = the default stream).  Tensors are dense row-major ("contiguous") except in the *_strided
  * entry points, which take explicit strides.  Launches are asynchronous on `stream`; the functions
- * never synchronise, never allocate and keep no state.
+ * never synchronise and never allocate.  The only state the library keeps is per device and is set
+ * on first use: the address of the fixed workspace of sma_attn_bwd_static_ws, and the verdict of a
+ * one-time check that the device serves copies from unaligned addresses (see sma_attn_fwd_bool_mask).
  * Return value: SMA_OK (0) or a negative SMA_ERR_* code; sma_strerror() names it.
  *
  * Each entry point cites the interface of the reference implementation that it stands in for
@@ -29,6 +31,7 @@ extern "C" {
 #define SMA_ERR_ALIGNMENT     -7   /* q/k/v/out not 16-byte aligned, or mask_packed/lse not 4-byte aligned */
 #define SMA_ERR_STRIDE        -8   /* a stride is negative, not a multiple of 8 elements, or too large */
 #define SMA_ERR_WORKSPACE     -9   /* B*H*N exceeds SMA_STATIC_WS_ROWS (sma_attn_bwd_static_ws only) */
+#define SMA_ERR_DEVICE       -10   /* the device does not serve loads from unaligned addresses (sma_device_check) */
 
 #define SMA_DTYPE_F16   0
 #define SMA_DTYPE_BF16  1
@@ -38,6 +41,23 @@ int sma_version(void);
 
 /* Static, never-NULL description of a return code. */
 const char *sma_strerror(int code);
+
+/* One-time check of the current device: are 8- and 16-byte loads from unaligned addresses served?
+ *
+ * The packers for rows that do not start 16-byte aligned and sma_attn_fwd_bool_mask read mask rows
+ * at whatever byte address they start.  ROCm runs compute queues in the unaligned-access mode of the
+ * memory pipeline, in which such loads are served; on a device where they are not, the results
+ * would be wrong without any fault.  The library therefore checks once per device, in the first
+ * call that depends on it (or in this one): a one-wavefront kernel on `stream`, whose verdict the
+ * call waits for - the one place where the library synchronises.  It cannot run while `stream` is
+ * being captured into a graph (the dependent calls then proceed unchecked): make the first call on
+ * a device outside capture.  Returns SMA_OK, or SMA_ERR_DEVICE when such loads are not served;
+ * sma_pack_mask then packs with byte loads (slower, same words) and sma_attn_fwd_bool_mask
+ * returns SMA_ERR_DEVICE (use sma_pack_mask + sma_attn_fwd).
+ *
+ * No counterpart in the reference.
+ */
+int sma_device_check(void *stream);
 
 /* Bit-pack a boolean attend-mask.
  *
@@ -65,7 +85,11 @@ int sma_pack_mask(const uint8_t *mask, uint32_t *packed, int B, int H, int N, vo
  * copied and nothing computed, which is what a block-structured mask (sliding window, block-sparse,
  * causal) needs; the reference's own skip (csrc/sparse_attention.cu:238-252) still loads the tile
  * (:211) and is taken per 64 query rows.  A map costs one pass over the packed words; make it once
- * for a mask that is used many times.  N <= 131072.
+ * for a mask that is used many times.  N <= 131072 (sma_tile_map, sma_pack_mask_map with a map and
+ * every entry point that takes a map return SMA_ERR_BAD_SHAPE beyond it, before anything is written).
+ *
+ * Word group 1 ("every bit set") is written for callers; the kernels of this library read word
+ * group 0 only.
  *
  * sma_pack_mask_map = sma_pack_mask followed by sma_tile_map on its output (tile_map may be NULL:
  * then it is sma_pack_mask).
@@ -255,16 +279,6 @@ int sma_attn_bwd_map_strided(const sma_tensor *dout, const sma_tensor *q, const 
                              const uint32_t *tile_map, const sma_tensor *dq, const sma_tensor *dk,
                              const sma_tensor *dv, float *delta_ws, int B, int H, int N, int D, float scale,
                              int dtype, void *stream);
-
-/* Yardstick for the MFMA roofline, used by the benchmark (not by the attention path): launches
- * `work_groups` work-groups of 12 wavefronts that each issue 8 * iters MFMAs of the kind the
- * attention kernels use (v_mfma_f32_32x32x16_f16), on operands that are all zero (random_operands
- * == 0) or random fp16 numbers.  Thread 0 of work-group g leaves in stamps[2g] the shader-clock
- * ticks and in stamps[2g+1] the 100 MHz ticks that its loop took (stamps: device memory, 2 *
- * work_groups int64).  Time the launch to get the sustained MFMA rate; the quotient of the two
- * stamps is the shader clock in units of 100 MHz.  No counterpart in the reference.
- */
-int sma_probe_mfma_stream(int random_operands, int iters, int work_groups, long long *stamps, void *stream);
 
 #ifdef __cplusplus
 }

@@ -190,13 +190,18 @@ def lse_ref(q: torch.Tensor, k: torch.Tensor, mask: torch.Tensor,
 
 
 def sparse_attention_bwd_ref(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: torch.Tensor,
-                             dout: torch.Tensor, scale: float | None = None):
+                             dout: torch.Tensor, scale: float | None = None, delta: torch.Tensor | None = None):
     """Gradients (dq, dk, dv) of sum(out * dout) for out = sparse_attention_ref(q, k, v, mask).
 
     The closed form of the reference's PyTorch fallback, python/sparse_attention.py:97-111:
     attn = softmax of the masked scaled scores (empty rows -> 0); dv = attn^T dout;
     dattn = dout v^T on kept entries; ds = attn * (dattn - rowsum(dattn * attn)) * scale;
     dq = ds k; dk = ds^T q.  Computed in the dtype given (tests pass fp32 or fp64 up-casts).
+
+    `delta` ([B,H,N,1]), if given, stands in for rowsum(dattn * attn).  The two are equal in exact
+    arithmetic when delta = sum_d dout * out (rowsum_j attn_ij dout_i.v_j = dout_i . out_i); a
+    backward that forms delta from an `out` already rounded to 16 bits, as every flash-style backward
+    does, computes exactly this function of that rounded `out`.
     """
     D = q.shape[-1]
     if scale is None:
@@ -206,7 +211,9 @@ def sparse_attention_bwd_ref(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, 
     attn = torch.nan_to_num(torch.softmax(s, dim=-1), nan=0.0)
     dv = torch.matmul(attn.transpose(-2, -1), dout)
     dattn = torch.matmul(dout, v.transpose(-2, -1)).masked_fill(~mask, 0.0)
-    ds = attn * (dattn - (dattn * attn).sum(dim=-1, keepdim=True)) * scale
+    if delta is None:
+        delta = (dattn * attn).sum(dim=-1, keepdim=True)
+    ds = attn * (dattn - delta) * scale
     dq = torch.matmul(ds, k)
     dk = torch.matmul(ds.transpose(-2, -1), q)
     return dq, dk, dv

@@ -3,9 +3,12 @@
 // random fp16 numbers, and the shader clock it gets while doing so.  The dense FP16 peak of the
 // data sheet (256 CUs x 4096 FLOP/clk x 2.4 GHz) assumes the top clock; the part lowers its clock
 // under a stream of MFMAs on real data, and this probe measures by how much on the GPU at hand.
-// No counterpart in the reference; used by bench.py, not by the attention path.
-#include "sma.h"
-#include "sma_internal.h"
+// No counterpart in the reference.  Benchmark infrastructure: built into libsma_probe.so, which only
+// bench.py and one test load; libsma_hip.so, the product, does not contain it.
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "mfma_probe.h"
 
 namespace sma {
 namespace {
@@ -68,10 +71,13 @@ __global__ __launch_bounds__(768) void mfma_stream_kernel(int random_operands, i
 
 extern "C" int sma_probe_mfma_stream(int random_operands, int iters, int work_groups, long long *stamps, void *stream)
 {
-    if (iters < 0 || work_groups < 0) return SMA_ERR_BAD_SHAPE;
-    if (work_groups == 0) return SMA_OK;
-    if (stamps == nullptr) return SMA_ERR_NULL_POINTER;
+    // a wavefront's loop is iters * 8 MFMAs of 32 cycles: the cap keeps a mistyped count from
+    // turning into a kernel that runs for minutes
+    if (iters < 0 || iters > SMA_PROBE_MAX_ITERS || work_groups < 0 || work_groups > 65536) return SMA_PROBE_ERR_RANGE;
+    if (work_groups == 0) return SMA_PROBE_OK;
+    if (stamps == nullptr) return SMA_PROBE_ERR_NULL;
+    // the kernel's last argument is a sink that is never written (see the kernel); any device address does
     hipLaunchKernelGGL(sma::mfma_stream_kernel, dim3((unsigned)work_groups), dim3(768), 0, static_cast<hipStream_t>(stream),
                        random_operands, iters, stamps, reinterpret_cast<float *>(stamps));
-    return hipGetLastError() == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
+    return hipGetLastError() == hipSuccess ? SMA_PROBE_OK : SMA_PROBE_ERR_LAUNCH;
 }

@@ -1,4 +1,4 @@
-"""In-tree build of the two native artefacts, for gfx950 only.
+"""In-tree build of the native artefacts, for gfx950 only.
 
 * ``libsma_hip.so``              the HIP kernels and the C ABI of ``include/sma.h``; compiled by
                                  ``hipcc --offload-arch=gfx950`` straight from ``csrc/*.hip``.
@@ -9,8 +9,12 @@
 The reference builds its extension through ``torch.utils.cpp_extension.CUDAExtension``
 (``setup.py:35-45``) or the JIT ``load`` (``run.py:118-135``); on ROCm both would first translate
 the sources with hipify, which is exactly what this build avoids: the sources are HIP already and
-go to the compilers as they are.  Both artefacts are written next to this file so that they
-travel with the source tree.
+go to the compilers as they are.
+
+* ``libsma_probe.so``            benchmark infrastructure, not the product: a pure stream of MFMAs that
+                                 ``bench.py`` times as a yardstick (``benchprobe/mfma_probe.hip``).
+
+All artefacts are written next to this file so that they travel with the source tree.
 """
 from __future__ import annotations
 
@@ -28,7 +32,9 @@ ROCM = os.environ.get("ROCM_PATH", "/opt/rocm")
 
 LIB_NAME = "libsma_hip.so"
 MODULE_NAME = "sparse_attn_cuda"
-HIP_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "pack_mask.hip", "capi.hip", "probe.hip"]
+HIP_SOURCES = ["attn_fwd.hip", "attn_bwd.hip", "pack_mask.hip", "capi.hip"]
+PROBE_DIR = os.path.join(HERE, "benchprobe")
+PROBE_LIB_NAME = "libsma_probe.so"
 GPU_ARCH = "gfx950"
 
 
@@ -52,17 +58,28 @@ def _run(cmd):
         raise RuntimeError(f"command failed with exit code {proc.returncode}: {' '.join(cmd)}")
 
 
+def probe_lib_path() -> str:
+    return os.path.join(HERE, PROBE_LIB_NAME)
+
+
+def hipcc_path() -> str:
+    return shutil.which("hipcc") or os.path.join(ROCM, "bin", "hipcc")
+
+
+# The device-code flags every HIP source of this package is compiled with (the ISA scan in the tests
+# compiles with the same list).
+HIPCC_FLAGS = [f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++17", "-fno-finite-math-only",
+               # keep the compiler from forming packed-FP32 VALU instructions
+               "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+               # the asynchronous-copy statements name m0, which they write, as clobbered; clang remarks
+               # on every reserved register in a clobber list
+               "-Wno-inline-asm",
+               f"-I{INCLUDE}", f"-I{CSRC}"]
+
+
 def build_hip_library() -> str:
-    hipcc = shutil.which("hipcc") or os.path.join(ROCM, "bin", "hipcc")
     out = lib_path()
-    cmd = [hipcc, f"--offload-arch={GPU_ARCH}", "-O3", "-std=c++17", "-fPIC", "-shared",
-           "-fno-finite-math-only",
-           # keep the compiler from forming packed-FP32 VALU instructions
-           "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
-           # the asynchronous-copy statements name m0, which they write, as clobbered; clang remarks
-           # on every reserved register in a clobber list
-           "-Wno-inline-asm",
-           f"-I{INCLUDE}", f"-I{CSRC}"]
+    cmd = [hipcc_path()] + HIPCC_FLAGS + ["-fPIC", "-shared"]
     cmd += [os.path.join(CSRC, s) for s in HIP_SOURCES]
     cmd += ["-o", out, f"-Wl,-rpath,{os.path.join(ROCM, 'lib')}", "-Wl,-soname," + LIB_NAME]
     _run(cmd)
@@ -90,9 +107,19 @@ def build_python_module() -> str:
     return out
 
 
+def build_probe_library() -> str:
+    out = probe_lib_path()
+    cmd = [hipcc_path()] + HIPCC_FLAGS + ["-fPIC", "-shared", f"-I{PROBE_DIR}",
+                                           os.path.join(PROBE_DIR, "mfma_probe.hip"), "-o", out,
+                                           f"-Wl,-rpath,{os.path.join(ROCM, 'lib')}", "-Wl,-soname," + PROBE_LIB_NAME]
+    _run(cmd)
+    return out
+
+
 def build_all() -> None:
     build_hip_library()
     build_python_module()
+    build_probe_library()
 
 
 if __name__ == "__main__":

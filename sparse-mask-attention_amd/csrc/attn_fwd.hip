@@ -148,16 +148,15 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
             mapw2 = (2 * qt + 1 < T) ? mapw + 2 * TW : mapw;
         }
     }
-    // The loads are issued whether there is a map or not (without one they read the first word of q,
-    // which exists and is aligned, and their result is dropped): a branch around them would give the registers a
-    // second definition on the other path, and between this statement and the one that waits for
-    // the loads nothing may touch them.
+    // The first map words are read here, with ordinary (scalar) loads, long before they are needed:
+    // the address arithmetic below covers their latency.
+    // (Without a map they read the first word of q, which exists, and the result is dropped: no
+    // branch, so the loads stay where they are written.  The words are combined only where the walk
+    // starts; the compiler puts its wait there.)
     const bool has_map = mapw != nullptr;
     const uint32_t *mapa = has_map ? mapw : reinterpret_cast<const uint32_t *>(a.q.p);
     const uint32_t *mapb = has_map ? mapw2 : reinterpret_cast<const uint32_t *>(a.q.p);
-    uint32_t live_w, live_w2;
-    asm volatile("s_load_dword %0, %2, 0x0\n\ts_load_dword %1, %3, 0x0"
-                 : "=&s"(live_w), "=&s"(live_w2) : "s"(mapa), "s"(mapb) : "memory");
+    const uint32_t first_w = mapa[0], first_w2 = mapb[0];
     const uint16_t *qb = slab(a.q, bi, hi);
     const uint16_t *kb = slab(a.k, bi, hi);
     const uint16_t *vb = slab(a.v, bi, hi);
@@ -447,9 +446,7 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         }
     }
     using std::integral_constant;
-    // the map word has had the whole address arithmetic above to arrive
-    asm volatile("s_waitcnt lgkmcnt(0)" : "+s"(live_w), "+s"(live_w2) :: "memory");
-    live_w = has_map ? (live_w | live_w2) : 0xffffffffu;
+    uint32_t live_w = has_map ? (first_w | first_w2) : 0xffffffffu;
     if ((T & 31) != 0 && TW == 1) live_w &= (1u << (T & 31)) - 1u;
     const int n_visits = TW == 1 ? __builtin_popcount(live_w) : T;
     // Walk over the set bits of the "live" words: `live_w` holds the bits of word `cur_w` that have

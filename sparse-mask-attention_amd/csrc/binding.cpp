@@ -140,7 +140,10 @@ bool bool_mask_supported(const torch::Tensor &q, const torch::Tensor &k, const t
     if (!((mask.size(0) == B || mask.size(0) == 1) && (mask.size(1) == H || mask.size(1) == 1) &&
           mask.size(2) == N && mask.size(3) == N))
         return false;
-    return true;
+    // the kernel copies mask rows from whatever byte address they start at: the library checks once
+    // per device that such copies are served (always, under ROCm); where not, pack_mask + forward
+    const c10::DeviceGuard guard(q.device());
+    return sma_device_check(c10::hip::getCurrentHIPStream(q.device().index()).stream()) == SMA_OK;
 }
 
 void forward_bool_mask(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,

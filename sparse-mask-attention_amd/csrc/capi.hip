@@ -77,6 +77,7 @@ const char *sma_strerror(int code)
     case SMA_ERR_ALIGNMENT:    return "misaligned pointer";
     case SMA_ERR_STRIDE:       return "bad stride: negative, not a multiple of 8 elements, or too large";
     case SMA_ERR_WORKSPACE:    return "problem too large for the library's static workspace";
+    case SMA_ERR_DEVICE:       return "the device does not serve loads from unaligned addresses";
     default:                   return "unknown error code";
     }
 }
@@ -100,9 +101,18 @@ int sma_tile_map(const uint32_t *mask_packed, uint32_t *tile_map, int B, int H, 
     return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
 }
 
+int sma_device_check(void *stream)
+{
+    return sma::unaligned_access_state(static_cast<hipStream_t>(stream)) == 0 ? SMA_ERR_DEVICE : SMA_OK;
+}
+
 int sma_pack_mask_map(const uint8_t *mask, uint32_t *packed, uint32_t *tile_map, int B, int H, int N,
                       void *stream)
 {
+    // what sma_tile_map would refuse is refused before anything is written
+    if (tile_map != nullptr && B >= 0 && H >= 0 &&
+        (N > 131072 || (long long)B * H * ((N + 63) / 64) >= (1ll << 31) || misaligned(tile_map, 4)))
+        return misaligned(tile_map, 4) ? SMA_ERR_ALIGNMENT : SMA_ERR_BAD_SHAPE;
     const int st = sma_pack_mask(mask, packed, B, H, N, stream);
     if (st != SMA_OK || tile_map == nullptr) return st;
     return sma_tile_map(packed, tile_map, B, H, N, stream);
@@ -237,6 +247,7 @@ int sma_attn_fwd_map_strided(const sma_tensor *q, const sma_tensor *k, const sma
     if ((long long)N * ((N + 31) / 32) * 4 >= (1ll << 32)) return SMA_ERR_BAD_SHAPE;
     if (misaligned(mask_packed, 4) || (lse && misaligned(lse, 4)) || (tile_map && misaligned(tile_map, 4)))
         return SMA_ERR_ALIGNMENT;
+    if (tile_map && N > 131072) return SMA_ERR_BAD_SHAPE;      // the limit of sma_tile_map, which makes the maps
     if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
 
     sma::AttnArgs a;
@@ -319,6 +330,8 @@ int sma_attn_fwd_bool_mask_map(const void *q, const void *k, const void *v, cons
     // N * N above is the tighter one)
     if (map_out && (N + 63) / 64 > 32 * 32) return SMA_ERR_BAD_SHAPE;
     if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
+    // mask rows start at any byte address: the kernel's 16-byte copies rely on the device serving them
+    if (sma::unaligned_access_state(static_cast<hipStream_t>(stream)) == 0) return SMA_ERR_DEVICE;
 
     sma::AttnArgs a;
     const sma_tensor t[4] = {dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D), dense(out, H, N, D)};
@@ -361,8 +374,14 @@ int sma_attn_bwd_static_ws(const void *dout, const void *q, const void *k, const
                            const float *lse, const uint32_t *mask_packed, void *dq, void *dk, void *dv,
                            int B, int H, int N, int D, float scale, int dtype, void *stream)
 {
-    if (B < 0 || H < 0 || N < 0) return SMA_ERR_BAD_SHAPE;
-    if ((long long)B * H * N > STATIC_WS_ROWS) return SMA_ERR_WORKSPACE;
+    // the cheap argument checks of sma_attn_bwd first, so that a bad call reports what is wrong with
+    // it and neither an empty nor an invalid call touches the workspace
+    if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
+    if (D != 32 && D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
+    if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
+    if (!isfinite(scale)) return SMA_ERR_SCALE;
+    if (B == 0 || H == 0 || N == 0) return SMA_OK;
+    if ((long long)B * H > STATIC_WS_ROWS || (long long)B * H * (long long)N > STATIC_WS_ROWS) return SMA_ERR_WORKSPACE;
     float *ws = static_workspace();
     if (ws == nullptr) return SMA_ERR_LAUNCH;
     // Both kernels run on `stream`, the first writes every entry the second reads: nothing has to

@@ -23,6 +23,10 @@
 // The loads are ordinary (temporal) ones.  Non-temporal loads make the packer alone 15 % faster in
 // a loop over the same mask, but the sequence pack -> attention, which is what a caller runs,
 // 8 % slower (measured on MI355X: 32.5 vs 29.7 us for B=16, H=12, N=512).
+#include <stdlib.h>
+
+#include <atomic>
+
 #include "sma_internal.h"
 
 namespace sma {
@@ -181,6 +185,65 @@ __global__ __launch_bounds__(PACK_THREADS) void pack_short_rows_kernel(const uin
     packed[row] = acc;
 }
 
+// Any N, byte loads only, one lane per output word: the packer for a device that does not serve
+// 8-byte loads from unaligned addresses (see unaligned_access_state below); several times slower
+// than the kernels above and never used where they work.
+__global__ __launch_bounds__(PACK_THREADS) void pack_bytewise_kernel(const uint8_t *__restrict__ mask,
+                                                                     uint32_t *__restrict__ packed,
+                                                                     long long words, int N, int nw)
+{
+    const long long idx = (long long)blockIdx.x * PACK_THREADS + threadIdx.x;
+    if (idx >= words) return;
+    const long long row = idx / nw;
+    const int w = (int)(idx - row * nw);
+    const uint8_t *src = mask + row * N + 32 * w;
+    const int n = N - 32 * w < 32 ? N - 32 * w : 32;
+    uint32_t acc = 0u;
+    for (int j = 0; j < n; ++j) acc |= (uint32_t)(src[j] != 0) << j;
+    packed[idx] = acc;
+}
+
+// ---- one-time check of the device: are 8- and 16-byte loads from unaligned addresses served? ----
+// The row packers above and the forward that reads the boolean mask load 8 bytes (into registers)
+// and 16 bytes (into LDS) from whatever address a mask row starts at.  ROCm runs compute queues in
+// the memory pipeline's unaligned-access mode, in which that is served; with the mode off the
+// hardware drops the low address bits and the results would be silently wrong.  One wavefront
+// writes a byte pattern, loads it back both ways from odd addresses and compares.
+constexpr int PROBE_BYTES = 1024 + 64;
+__device__ __align__(16) unsigned char unaligned_probe_src[PROBE_BYTES];
+__device__ int unaligned_probe_verdict;
+
+__device__ __forceinline__ uint32_t probe_byte(uint32_t i) { return (i * 37u + 11u) & 0xffu; }
+
+__global__ __launch_bounds__(64) void unaligned_probe_kernel(unsigned char *src, int *verdict)
+{
+    __shared__ __attribute__((aligned(16))) unsigned char landing[1024];
+    const uint32_t lane = threadIdx.x;
+    for (uint32_t i = lane * 17u; i < lane * 17u + 17u; ++i) src[i] = (unsigned char)probe_byte(i);
+    __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "agent");
+    __builtin_amdgcn_s_barrier();
+    bool ok = true;
+    // 8 bytes into registers from an address that is 3 mod 8
+    {
+        uint64_t v;
+        const unsigned char *p = src + 3 + 8 * lane;
+        asm volatile("global_load_dwordx2 %0, %1, off\n\ts_waitcnt vmcnt(0)" : "=v"(v) : "v"(p) : "memory");
+        for (uint32_t b = 0; b < 8; ++b) ok &= ((v >> (8 * b)) & 0xffu) == probe_byte(3 + 8 * lane + b);
+    }
+    // 16 bytes into LDS from an address that is 5 mod 16 (lane i's bytes land at 16 * i)
+    {
+        const uint32_t lds = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) unsigned char *)landing;
+        const uint32_t voff = 5u + 16u * lane;
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2\n\ts_waitcnt vmcnt(0)"
+                     :: "s"(lds), "v"(voff), "s"(src) : "memory", "m0");
+        __builtin_amdgcn_fence(__ATOMIC_SEQ_CST, "workgroup");
+        __builtin_amdgcn_s_barrier();
+        for (uint32_t b = 0; b < 16; ++b) ok &= landing[16 * lane + b] == probe_byte(5 + 16 * lane + b);
+    }
+    const bool all_ok = __builtin_amdgcn_ballot_w64(!ok) == 0ull;
+    if (lane == 0) *verdict = all_ok ? 1 : 2;
+}
+
 // Tile map of a packed mask: for every (slab, block of 64 query rows) one bit per 64-key tile that
 // says "some mask bit of this 64 x 64 block is set" (word group 0) and one that says "every bit of
 // the block is set" (word group 1; only rows and columns below N count).  Layout
@@ -235,12 +298,51 @@ hipError_t launch_tile_map(const uint32_t *packed, uint32_t *map, long long slab
     return hipGetLastError();
 }
 
+int unaligned_access_state(hipStream_t stream)
+{
+    static std::atomic<int> cached[64];      // 0 = not checked yet, 1 = served, 2 = not served
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return -1;
+    const int known = cached[dev].load(std::memory_order_acquire);
+    if (known != 0) return known == 1 ? 1 : 0;
+    // not under graph capture: the check reads its verdict back and waits for it
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(stream, &cap) != hipSuccess || cap != hipStreamCaptureStatusNone) {
+        (void)hipGetLastError();
+        return -1;
+    }
+    int verdict = 0;
+    const char *forced = getenv("SMA_ASSUME_NO_UNALIGNED_ACCESS");      // for tests of the fallbacks
+    if (forced != nullptr && forced[0] == '1') {
+        verdict = 2;
+    } else {
+        void *src = nullptr, *res = nullptr;
+        if (hipGetSymbolAddress(&src, HIP_SYMBOL(unaligned_probe_src)) != hipSuccess ||
+            hipGetSymbolAddress(&res, HIP_SYMBOL(unaligned_probe_verdict)) != hipSuccess)
+            return -1;
+        hipLaunchKernelGGL(unaligned_probe_kernel, dim3(1), dim3(64), 0, stream, static_cast<unsigned char *>(src),
+                           static_cast<int *>(res));
+        if (hipGetLastError() != hipSuccess) return -1;
+        if (hipMemcpyAsync(&verdict, res, sizeof(int), hipMemcpyDeviceToHost, stream) != hipSuccess) return -1;
+        if (hipStreamSynchronize(stream) != hipSuccess) return -1;
+        if (verdict != 1 && verdict != 2) return -1;
+    }
+    cached[dev].store(verdict, std::memory_order_release);
+    return verdict == 1 ? 1 : 0;
+}
+
 hipError_t launch_pack_mask(const uint8_t *mask, uint32_t *packed, long long rows, int N,
                             hipStream_t stream)
 {
     if (rows == 0 || N == 0) return hipSuccess;
     const int nw = (N + 31) / 32;
     const bool flat = (N % 32 == 0) && ((reinterpret_cast<uintptr_t>(mask) & 15u) == 0);
+    if (!flat && N >= 8 && unaligned_access_state(stream) == 0) {
+        const long long words = rows * nw;
+        const unsigned grid = (unsigned)((words + PACK_THREADS - 1) / PACK_THREADS);
+        hipLaunchKernelGGL(pack_bytewise_kernel, dim3(grid), dim3(PACK_THREADS), 0, stream, mask, packed, words, N, nw);
+        return hipGetLastError();
+    }
     if (flat) {
         const long long n_chunks = rows * (long long)N / 16;
         const long long per_block = (long long)PACK_THREADS * PACK_UNROLL;

@@ -95,6 +95,11 @@ hipError_t launch_attn_fwd(const AttnArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_attn_bwd(const AttnBwdArgs &a, bool bf16, hipStream_t stream);
 hipError_t launch_pack_mask(const uint8_t *mask, uint32_t *packed, long long rows, int N,
                             hipStream_t stream);
+// Whether the current device serves 8- and 16-byte loads from unaligned addresses (the row packers
+// and the forward that reads the boolean mask depend on it): 1 yes, 0 no, -1 not known (the
+// one-time check could not run because `stream` is being captured into a graph, or failed).  The
+// first call per device launches a one-wavefront check on `stream` and waits for it.
+int unaligned_access_state(hipStream_t stream);
 // tile map [slabs, ceil(N/64), 2, ceil(ceil(N/64)/32)] of packed words [slabs, N, ceil(N/32)]
 hipError_t launch_tile_map(const uint32_t *packed, uint32_t *map, long long slabs, int N, hipStream_t stream);
 

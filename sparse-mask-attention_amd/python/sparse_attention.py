@@ -42,7 +42,8 @@ What differs from the reference, on purpose:
   which 64 x 64 blocks of the mask hold a set bit; given as ``tile_map=`` together with
   ``mask_packed=`` the forward neither loads nor computes the key tiles that hold none (the
   reference skips such a tile only after loading it, ``csrc/sparse_attention.cu:211,238-252``).
-  Worth it for a mask that is used many times; ``tile_map`` returns None when no block is empty.
+  Worth it for a mask that is used many times; ``tile_map`` returns None when too few visits would
+  disappear for the walk to pay.
 * ``.backward()`` works.  The reference calls a ``sparse_attn_cuda.backward`` that was never
   written (:91-94); here that function exists (two HIP kernels, dQ and dK/dV, from the saved
   log-sum-exp and the packed mask).  ``backward_recompute`` states the same gradients with PyTorch
@@ -110,8 +111,8 @@ class SparseAttentionFunction(Function):
     """forward = fused HIP kernel (saves LSE); backward = the HIP dQ and dK/dV kernels.
 
     ``mask_packed`` may be None: the mask is then read as it is by the one-launch forward, which
-    leaves the packed words and the tile map the backward uses as by-products, or packed first
-    where that kernel does not apply."""
+    leaves the packed words the backward uses (and, with ``tile_map=True``, the mask's tile map) as
+    by-products, or packed first where that kernel does not apply."""
 
     @staticmethod
     def forward(ctx, q, k, v, mask_packed, mask_bool, scale, seq_len, tile_map=None):
@@ -125,17 +126,23 @@ class SparseAttentionFunction(Function):
             if sparse_attn_cuda.bool_mask_supported(q, k, v, mask_bool):
                 mask_packed = torch.empty(mask_bool.shape[0], mask_bool.shape[1], N, (N + 31) // 32,
                                           device=q.device, dtype=torch.int32)
-                # the same launch leaves the mask's tile map behind: the backward visits only the
-                # blocks that hold something
-                T = (N + 63) // 64
-                tile_map = torch.empty(mask_bool.shape[0], mask_bool.shape[1], T, 2, (T + 31) // 32,
-                                       device=q.device, dtype=torch.int32)
+                # tile_map=True: the caller says the mask has empty 64 x 64 blocks; the same launch
+                # then leaves the mask's tile map behind and the backward visits only the blocks
+                # that hold something.  Not by default: a mask without empty blocks (any random one)
+                # would pay for a by-product that nothing can use.
+                if tile_map is True:
+                    T = (N + 63) // 64
+                    tile_map = torch.empty(mask_bool.shape[0], mask_bool.shape[1], T, 2, (T + 31) // 32,
+                                           device=q.device, dtype=torch.int32)
+                else:
+                    tile_map = None
                 sparse_attn_cuda.forward_bool_mask(q, k, v, mask_bool, out, lse, scale, True, mask_packed, tile_map)
                 ctx.save_for_backward(q, k, v, out, lse, mask_packed)
                 ctx.scale = scale
                 ctx.tile_map = tile_map
                 return out
             mask_packed = pack_mask(mask_bool)
+            tile_map = sparse_attn_cuda.tile_map(mask_packed) if tile_map is True else None
         sparse_attn_cuda.forward(q, k, v, mask_packed, out, lse, scale, True, tile_map)
         ctx.save_for_backward(q, k, v, out, lse, mask_packed)
         ctx.scale = scale
@@ -224,11 +231,15 @@ def sparse_attention(q, k, v, mask, mask_packed=None, tile_map=None):
 
     ``mask_packed`` (optional, not in the reference): the result of ``pack_mask(mask)`` kept from an
     earlier call with the same mask; packing (as much HBM traffic as the attention itself at
-    N = 512) is then skipped and ``mask`` may be None.  ``tile_map`` (optional, with ``mask_packed``):
+    N = 512) is then skipped and ``mask`` may be None.  ``tile_map`` (optional): with ``mask_packed``,
     the result of ``tile_map(mask_packed)``; key tiles in which the mask keeps nothing are skipped.
+    With a bool ``mask`` under autograd, ``tile_map=True`` says that the mask has empty 64 x 64 blocks:
+    the forward then leaves the map behind for the backward (about 1 us at N = 512; off by default,
+    because a mask without empty blocks gains nothing from it).
     """
     _check_inputs(q, k, v, mask, mask_packed)
-    assert tile_map is None or mask_packed is not None, "tile_map belongs to a mask_packed"
+    assert tile_map is None or tile_map is True or mask_packed is not None, "a tile_map tensor belongs to a mask_packed"
+    assert not (tile_map is True and mask_packed is not None), "with mask_packed, pass the result of tile_map(mask_packed)"
     _require_ext(q)
     if not (torch.is_grad_enabled() and (q.requires_grad or k.requires_grad or v.requires_grad)):
         # nothing will be differentiated: no LSE, and the mask can be read without packing it
@@ -251,6 +262,8 @@ def sparse_attention(q, k, v, mask, mask_packed=None, tile_map=None):
 def sparse_attention_func(q, k, v, mask, mask_packed=None, tile_map=None):
     """Inference-only variant of :func:`sparse_attention`: no autograd graph, no LSE."""
     _check_inputs(q, k, v, mask, mask_packed)
+    if tile_map is True:        # a hint for the backward only
+        tile_map = None
     assert tile_map is None or mask_packed is not None, "tile_map belongs to a mask_packed"
     _require_ext(q)
     D = q.shape[-1]
@@ -290,20 +303,28 @@ def pack_mask(mask: torch.Tensor) -> torch.Tensor:
     return sparse_attn_cuda.pack_mask(mask)
 
 
-def tile_map(mask_packed: torch.Tensor):
+def tile_map(mask_packed: torch.Tensor, min_skip: float = 0.25):
     """Occupancy of the 64 x 64 blocks of a packed mask, for ``sparse_attention(..., mask_packed=,
     tile_map=)``: int32 ``[B, H, T, 2, ceil(T/32)]`` with T = ceil(N/64); per block of 64 query rows
-    one bit per 64-key tile "some entry kept", then one bit per tile "every entry kept".  Returns
-    None when every block holds a kept entry (nothing could be skipped).  Synchronises with the
+    one bit per 64-key tile "some entry kept", then one bit per tile "every entry kept".
+
+    Returns None when the map would not pay: the forward walks the key tiles per 128 query rows (two
+    row blocks), and below ``min_skip`` (default a quarter) of those visits saved the walk costs what
+    it saves (a causal mask at N = 256 skips 6 of 32 visits per head and runs no faster with the
+    map).  ``min_skip=0`` returns the map whenever a single visit disappears.  Synchronises with the
     device once, to look at that; meant to be called once for a mask that is used many times."""
     _require_ext(mask_packed)
     tm = sparse_attn_cuda.tile_map(mask_packed)
     T = tm.shape[2]
     live = tm[:, :, :, 0, :]
-    every = torch.full((live.shape[-1],), -1, dtype=torch.int32, device=tm.device)
-    if T % 32:
-        every[-1] = (1 << (T % 32)) - 1
-    return None if bool((live == every).all()) else tm
+    if T % 2:                                   # the last work-group has one row block only
+        live = torch.cat([live, torch.zeros_like(live[:, :, :1])], dim=2)
+    pairs = live[:, :, 0::2] | live[:, :, 1::2]             # what a work-group of 128 rows visits
+    bits = (pairs.unsqueeze(-1) >> torch.arange(32, device=tm.device, dtype=torch.int32)) & 1
+    visited = int(bits.sum().item())
+    total = pairs.shape[0] * pairs.shape[1] * pairs.shape[2] * T
+    skipped = total - visited
+    return tm if skipped > 0 and skipped >= min_skip * total else None
 
 
 def generate_random_sparse_mask(B, H, N, sparsity=0.75, device="cuda"):

@@ -17,11 +17,13 @@ SMA_ERR_LAUNCH = -6
 SMA_ERR_ALIGNMENT = -7
 SMA_ERR_STRIDE = -8
 SMA_ERR_WORKSPACE = -9
+SMA_ERR_DEVICE = -10
 SMA_STATIC_WS_ROWS = 1 << 20
 SMA_DTYPE_F16 = 0
 SMA_DTYPE_BF16 = 1
 
 _lib = None
+_probe = None
 
 
 class SmaTensor(ctypes.Structure):
@@ -60,8 +62,8 @@ def load():
         lib.sma_pack_mask_map.argtypes = [vp, vp, vp, ci, ci, ci, vp]
         lib.sma_attn_fwd_map.restype = ci
         lib.sma_attn_fwd_map.argtypes = [vp, vp, vp, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
-        lib.sma_probe_mfma_stream.restype = ci
-        lib.sma_probe_mfma_stream.argtypes = [ci, ci, ci, vp, vp]
+        lib.sma_device_check.restype = ci
+        lib.sma_device_check.argtypes = [vp]
         lib.sma_attn_bwd_map.restype = ci
         lib.sma_attn_bwd_map.argtypes = [vp] * 12 + [ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_bwd_static_ws.restype = ci
@@ -81,6 +83,20 @@ def load():
         lib.sma_attn_fwd_bool_mask_map.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         _lib = lib
     return _lib
+
+
+def load_probe():
+    """libsma_probe.so, the benchmark's MFMA yardstick (benchprobe/mfma_probe.h): not the product."""
+    global _probe
+    if _probe is None:
+        path = os.path.join(os.path.dirname(LIB), "libsma_probe.so")
+        if not os.path.exists(path):
+            raise RuntimeError(f"{path} is not built; run __graft_entry__.build()")
+        lib = ctypes.CDLL(path)
+        lib.sma_probe_mfma_stream.restype = ctypes.c_int
+        lib.sma_probe_mfma_stream.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+        _probe = lib
+    return _probe
 
 
 def _stream():

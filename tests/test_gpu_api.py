@@ -380,8 +380,9 @@ def test_inference_entry_point_reads_the_bool_mask_itself(sa, dev, monkeypatch):
 
 
 def test_autograd_from_a_bool_mask_with_empty_blocks_uses_the_map_and_changes_nothing(sa, dev):
-    """With a bool mask the one-launch forward hands the backward the packed words and the tile map;
-    the gradients are those of the path that packs first and walks every tile, bit for bit."""
+    """With a bool mask the one-launch forward hands the backward the packed words and, when the caller
+    says `tile_map=True`, the tile map; either way the gradients are those of the path that packs
+    first and walks every tile, bit for bit."""
     g = torch.Generator().manual_seed(21)
     B, H, N = 2, 3, 320
     blocks = torch.rand(B, H, 5, 5, generator=g) < 0.3
@@ -389,13 +390,19 @@ def test_autograd_from_a_bool_mask_with_empty_blocks_uses_the_map_and_changes_no
     q, k, v, do = (torch.randn(B, H, N, 64, generator=g).half().to(dev) for _ in range(4))
     md = mask.to(dev)
     grads = []
-    for kw in ({}, {"mask_packed": sa.pack_mask(md)}):
+    for kw in ({}, {"tile_map": True}, {"mask_packed": sa.pack_mask(md)}):
         leaves = [t.clone().requires_grad_(True) for t in (q, k, v)]
-        out = sa.sparse_attention(*leaves, None if kw else md, **kw)
+        out = sa.sparse_attention(*leaves, None if "mask_packed" in kw else md, **kw)
         out.backward(do)
         grads.append([out.detach()] + [t.grad for t in leaves])
-    for a, b in zip(*grads):
-        assert torch.equal(a, b)
+    for other in grads[1:]:
+        for a, b in zip(grads[0], other):
+            assert torch.equal(a, b)
+    # tile_map=True really hands a map to the backward, the default hands none
+    for kw, has_map in (({}, False), ({"tile_map": True}, True)):
+        leaves = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        out = sa.sparse_attention(*leaves, md, **kw)
+        assert (getattr(out.grad_fn, "tile_map", None) is not None) == has_map
     wanted = O.sparse_attention_bwd_ref(q.float().cpu(), k.float().cpu(), v.float().cpu(), mask, do.float().cpu())
     for got, want in zip(grads[0][1:], wanted):
         assert torch.allclose(got.float().cpu(), want, atol=1e-4 + 1e-2 * want.abs().max().item(), rtol=1e-2)
@@ -405,18 +412,20 @@ def test_mfma_stream_probe_runs_and_reports_a_clock(dev):
     """The benchmark's yardstick kernel: finishes, and the two tick counts it leaves give a shader
     clock that a GPU of this kind can have."""
     import _capi
-    lib = _capi.load()
+    lib = _capi.load_probe()
     groups = 8
     stamps = torch.zeros(2 * groups, dtype=torch.int64, device=dev)
     for random_operands in (0, 1):
-        assert lib.sma_probe_mfma_stream(random_operands, 2000, groups, stamps.data_ptr(), None) == _capi.SMA_OK
+        assert lib.sma_probe_mfma_stream(random_operands, 2000, groups, stamps.data_ptr(), None) == 0
         torch.cuda.synchronize()
         st = stamps.view(groups, 2).double().cpu()
         assert (st > 0).all()
         ghz = (st[:, 0] / (st[:, 1] * 10.0)).mean().item()
         assert 0.3 < ghz < 3.0, ghz
-    assert lib.sma_probe_mfma_stream(1, 10, 0, None, None) == _capi.SMA_OK
-    assert lib.sma_probe_mfma_stream(1, 10, 4, None, None) == _capi.SMA_ERR_NULL_POINTER
+    assert lib.sma_probe_mfma_stream(1, 10, 0, None, None) == 0
+    assert lib.sma_probe_mfma_stream(1, 10, 4, None, None) == -1          # stamps missing
+    assert lib.sma_probe_mfma_stream(1, (1 << 22) + 1, 4, stamps.data_ptr(), None) == -2     # iteration cap
+    assert not hasattr(_capi.load(), "sma_probe_mfma_stream")             # not part of the product library
 
 
 def test_command_line_harness_acceptance_run_and_sweeps(dev, capsys):

@@ -51,8 +51,8 @@ def _mask(rng, g, Bm, Hm, N):
     return m
 
 
-@pytest.mark.parametrize("seed", range(40))
-def test_random_configuration(dev, seed):
+def _draw(seed):
+    """The configuration that belongs to a seed: (D, dtype, B, H, N, Bm, Hm, scale, layouts, q, k, v, do, mask)."""
     rng = random.Random(seed)
     g = torch.Generator().manual_seed(seed)
     D = rng.choice([32, 64, 128])
@@ -64,6 +64,49 @@ def test_random_configuration(dev, seed):
     layouts = [rng.choice(["dense", "bnhd", "hbnd", "padded"]) for _ in range(8)]
     q, k, v, do = [torch.randn(B, H, N, D, generator=g).to(dtype) for _ in range(4)]
     mask = _mask(rng, g, Bm, Hm, N)
+    return D, dtype, B, H, N, Bm, Hm, scale, layouts, q, k, v, do, mask
+
+
+# Seeds outside the 40 below on which dq misses the ordinary bar (found by drawing 59 360 more of
+# them once; all have N = 7, almost all are bf16): kept as a fixed list.
+FLOOR_SEEDS = [8315, 15725, 23526, 54200]
+
+
+@pytest.mark.parametrize("seed", FLOOR_SEEDS)
+def test_backward_accuracy_floor_is_the_rounding_of_out(dev, seed):
+    """The backward forms delta = sum_d dout * out from the forward's 16-bit `out`, so dS = p * (dP -
+    delta) carries an absolute error of about (rounding of out) x |dout| whatever the size of the
+    gradient; where the true gradient nearly cancels, that floor is what misses the ordinary bar.
+    Pinned here: on those seeds the kernels agree with the closed form evaluated in fp32 with delta
+    taken from the SAME rounded `out` to 1e-4 (plus the rounding of the 16-bit result itself), while
+    dv, which does not involve delta, meets the ordinary bar.  If this failed, the misses would
+    be a defect of the kernels and not the floor."""
+    D, dtype, B, H, N, Bm, Hm, scale, layouts, q, k, v, do, mask = _draw(seed)
+    tag = f"seed {seed}: D{D} {dtype} B{B} H{H} N{N} mask[{Bm},{Hm}] scale {scale}"
+    print(tag, flush=True)
+    qd, kd, vd, dod = (t.to(dev) for t in (q, k, v, do))
+    packed = _capi.pack_mask(mask.to(dev))
+    out, lse = _capi.attn_fwd_strided(qd, kd, vd, packed, scale=scale, want_lse=True)
+    dq, dk, dv, _ = _capi.attn_bwd_strided(dod, qd, kd, vd, out, lse, packed, scale=scale)
+    torch.cuda.synchronize()
+    full = mask.expand(B, H, N, N)
+    delta = (do.float() * out.float().cpu()).sum(dim=-1, keepdim=True)
+    refs = O.sparse_attention_bwd_ref(q.float(), k.float(), v.float(), full, do.float(), scale=scale, delta=delta)
+    out_eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -10          # rounding of the stored gradient
+    for name, got, want in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
+        err = (got.float().cpu() - want).abs()
+        assert (err <= 1e-4 + out_eps * want.abs()).all(), f"{name} {tag}: max err {err.max():.3e}"
+    # and against the delta-free oracle the ordinary bar holds for dv and fails, if at all, for dq / dk only
+    plain = O.sparse_attention_bwd_ref(q.float(), k.float(), v.float(), full, do.float(), scale=scale)
+    sharp = max(1.0, abs(scale) * math.sqrt(D)) if scale is not None else 1.0
+    want = plain[2]
+    bound = 1e-4 + sharp * (1e-2 * want.abs().max() + RTOL[dtype] * want.abs())
+    assert ((dv.float().cpu() - want).abs() <= bound).all(), f"dv {tag}"
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_random_configuration(dev, seed):
+    D, dtype, B, H, N, Bm, Hm, scale, layouts, q, k, v, do, mask = _draw(seed)
     tag = f"seed {seed}: D{D} {dtype} B{B} H{H} N{N} mask[{Bm},{Hm}] scale {scale} layouts {layouts}"
     print(tag, flush=True)
 

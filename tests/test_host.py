@@ -27,7 +27,7 @@ def test_library_exports_every_declared_symbol(capi):
         assert hasattr(capi, name), f"{name} is declared in sma.h but not exported"
     assert capi.sma_version() >= 100
     assert capi.sma_strerror(0) == b"ok"
-    for code in range(-9, 0):
+    for code in range(-10, 0):
         assert capi.sma_strerror(code) not in (b"ok", b"unknown error code")
     assert capi.sma_strerror(-99) == b"unknown error code"
 
@@ -54,6 +54,24 @@ def test_argument_validation_needs_no_gpu(capi):
     assert call(B=0) == _capi.SMA_OK and call(N=0) == _capi.SMA_OK          # empty problem: nothing to do
     assert call(B=1 << 20, H=1 << 12, N=64) == _capi.SMA_ERR_BAD_SHAPE      # index range
     assert call(B=1, H=1, N=200000) == _capi.SMA_ERR_BAD_SHAPE              # packed mask of one (b,h) beyond 4 GiB
+
+    # a tile map is refused beyond the size the library can make one for, by every entry point that
+    # takes one and before anything is written (N = 140000 is inside the packed-mask limit)
+    assert capi.sma_attn_fwd_map(p, p, p, p, p, p, None, 1, 1, 140000, 64, 0.125, 0, None) == _capi.SMA_ERR_BAD_SHAPE
+    assert capi.sma_attn_bwd_map(p, p, p, p, p, p, p, p, p, p, p, p, 1, 1, 140000, 64, 0.125, 0, None) == _capi.SMA_ERR_BAD_SHAPE
+    assert capi.sma_pack_mask_map(p, p, p, 1, 1, 140000, None) == _capi.SMA_ERR_BAD_SHAPE
+    assert capi.sma_tile_map(p, p, 1, 1, 140000, None) == _capi.SMA_ERR_BAD_SHAPE
+    # the backward with the library's own workspace: what is wrong with the arguments is reported as
+    # such, whatever the size; an empty problem is a no-op; only a valid call can be too large
+    ws = capi.sma_attn_bwd_static_ws
+    big = (1 << 10, 1 << 5, 64)            # 2^21 rows
+    assert ws(*([p] * 10), *big, 96, 0.125, 0, None) == _capi.SMA_ERR_HEAD_DIM
+    assert ws(*([p] * 10), *big, 64, 0.125, 7, None) == _capi.SMA_ERR_DTYPE
+    assert ws(*([p] * 10), *big, 64, float("nan"), 0, None) == _capi.SMA_ERR_SCALE
+    assert ws(*([p] * 10), -1, 1, 64, 64, 0.125, 0, None) == _capi.SMA_ERR_BAD_SHAPE
+    assert ws(*([p] * 10), 0, 1, 64, 64, 0.125, 0, None) == _capi.SMA_OK
+    assert ws(*([p] * 10), *big, 64, 0.125, 0, None) == _capi.SMA_ERR_WORKSPACE
+    assert ws(*([p] * 10), 1 << 30, 1 << 30, 1 << 30, 64, 0.125, 0, None) == _capi.SMA_ERR_WORKSPACE   # no overflow on the way
 
     # strided entry point: the descriptor is checked before anything is launched
     fs = capi.sma_attn_fwd_strided

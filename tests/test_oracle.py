@@ -241,6 +241,28 @@ def test_backward_all_true_mask_equals_dense_sdpa_autograd():
         assert torch.allclose(got, ref, atol=1e-10, rtol=1e-8)
 
 
+def test_backward_with_delta_given_is_the_delta_free_form():
+    """`delta=` only replaces rowsum(dattn * attn): with delta = sum_d dout * out of the exact `out` the
+    gradients are those of the delta-free form (fp64), and a perturbed delta moves dq and dk by
+    exactly attn * (-perturbation) * scale pushed through the last two products, dv not at all."""
+    q, k, v, do, mask = _bwd_case(2, 2, 33, seed=55)
+    scale = 0.21
+    out = O.sparse_attention_ref(q, k, v, mask, scale=scale)
+    delta = (do * out).sum(dim=-1, keepdim=True)
+    plain = O.sparse_attention_bwd_ref(q, k, v, mask, do, scale=scale)
+    given = O.sparse_attention_bwd_ref(q, k, v, mask, do, scale=scale, delta=delta)
+    for a, b in zip(plain, given):
+        assert torch.allclose(a, b, atol=1e-12, rtol=1e-10)
+    eps = torch.randn(2, 2, 33, 1, generator=torch.Generator().manual_seed(56), dtype=torch.float64) * 1e-3
+    moved = O.sparse_attention_bwd_ref(q, k, v, mask, do, scale=scale, delta=delta + eps)
+    s = (q @ k.transpose(-1, -2)) * scale
+    attn = torch.nan_to_num(torch.softmax(s.masked_fill(~mask, float("-inf")), dim=-1), nan=0.0)
+    dds = attn * (-eps) * scale
+    assert torch.allclose(moved[0] - plain[0], dds @ k, atol=1e-12)
+    assert torch.allclose(moved[1] - plain[1], dds.transpose(-1, -2) @ q, atol=1e-12)
+    assert torch.equal(moved[2], plain[2])
+
+
 # ---------------------------------------------------------------------------
 # tile map
 # ---------------------------------------------------------------------------

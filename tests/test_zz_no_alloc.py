@@ -36,6 +36,26 @@ def test_two_calls_in_a_row_match_the_workspace_entry_point(dev, dtype):
             assert torch.equal(g, w), f"{name} differs at B={B} H={H} N={N} D={D}"
 
 
+def test_calls_allocate_no_device_memory(dev):
+    """What the entry point is for: after the first call on a device (which looks the array's address
+    up), a call leaves the device's free memory as it found it."""
+    args = _problem(2, 2, 200, 64, torch.float16, 11, dev)
+    lib = _capi.load()
+    dq, dk, dv = (torch.empty_like(args[1]) for _ in range(3))
+    p = [t.data_ptr() for t in args] + [dq.data_ptr(), dk.data_ptr(), dv.data_ptr()]
+    call = lambda: lib.sma_attn_bwd_static_ws(*p, 2, 2, 200, 64, 0.125, _capi.SMA_DTYPE_F16, None)
+    assert call() == _capi.SMA_OK
+    torch.cuda.synchronize()
+    first = dq.clone()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        assert call() == _capi.SMA_OK
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    assert torch.equal(dq, first)
+
+
 def test_static_workspace_limit_and_empty_problem(dev):
     lib = _capi.load()
     args = _problem(1, 1, 64, 64, torch.float16, 7, dev)
