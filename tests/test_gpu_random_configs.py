@@ -74,13 +74,14 @@ FLOOR_SEEDS = [8315, 15725, 23526, 54200]
 
 @pytest.mark.parametrize("seed", FLOOR_SEEDS)
 def test_backward_accuracy_floor_is_the_rounding_of_out(dev, seed):
-    """The backward forms delta = sum_d dout * out from the forward's 16-bit `out`, so dS = p * (dP -
-    delta) carries an absolute error of about (rounding of out) x |dout| whatever the size of the
-    gradient; where the true gradient nearly cancels, that floor is what misses the ordinary bar.
-    Pinned here: on those seeds the kernels agree with the closed form evaluated in fp32 with delta
-    taken from the SAME rounded `out` to 1e-4 (plus the rounding of the 16-bit result itself), while
-    dv, which does not involve delta, meets the ordinary bar.  If this failed, the misses would
-    be a defect of the kernels and not the floor."""
+    """The backward forms delta = sum_d dout * out from the forward's 16-bit `out` (as every flash-style
+    backward does), so dS = p * (dP - delta) carries an absolute error of about (rounding of out) x
+    |dout| whatever the size of the gradient; where the true gradient nearly cancels, that floor is
+    what misses the ordinary bar.  Pinned here on the seeds that miss it: against the oracle's closed
+    form with delta taken from the SAME rounded `out` (`delta=`, pinned in test_oracle.py) the kernels
+    meet HALF the ordinary bar for dq, dk and dv (measured: at most 0.26 of it), where against the
+    delta-free form dq or dk are at 1.04 to 14.9 times the bar.  If the misses had another cause,
+    changing nothing but delta in the oracle would not remove them."""
     D, dtype, B, H, N, Bm, Hm, scale, layouts, q, k, v, do, mask = _draw(seed)
     tag = f"seed {seed}: D{D} {dtype} B{B} H{H} N{N} mask[{Bm},{Hm}] scale {scale}"
     print(tag, flush=True)
@@ -90,18 +91,19 @@ def test_backward_accuracy_floor_is_the_rounding_of_out(dev, seed):
     dq, dk, dv, _ = _capi.attn_bwd_strided(dod, qd, kd, vd, out, lse, packed, scale=scale)
     torch.cuda.synchronize()
     full = mask.expand(B, H, N, N)
+    sharp = max(1.0, abs(scale) * math.sqrt(D)) if scale is not None else 1.0
     delta = (do.float() * out.float().cpu()).sum(dim=-1, keepdim=True)
     refs = O.sparse_attention_bwd_ref(q.float(), k.float(), v.float(), full, do.float(), scale=scale, delta=delta)
-    out_eps = 2.0 ** -8 if dtype == torch.bfloat16 else 2.0 ** -10          # rounding of the stored gradient
-    for name, got, want in zip(("dq", "dk", "dv"), (dq, dk, dv), refs):
-        err = (got.float().cpu() - want).abs()
-        assert (err <= 1e-4 + out_eps * want.abs()).all(), f"{name} {tag}: max err {err.max():.3e}"
-    # and against the delta-free oracle the ordinary bar holds for dv and fails, if at all, for dq / dk only
     plain = O.sparse_attention_bwd_ref(q.float(), k.float(), v.float(), full, do.float(), scale=scale)
-    sharp = max(1.0, abs(scale) * math.sqrt(D)) if scale is not None else 1.0
-    want = plain[2]
-    bound = 1e-4 + sharp * (1e-2 * want.abs().max() + RTOL[dtype] * want.abs())
-    assert ((dv.float().cpu() - want).abs() <= bound).all(), f"dv {tag}"
+    worst_plain = 0.0
+    for name, got, want, want_plain in zip(("dq", "dk", "dv"), (dq, dk, dv), refs, plain):
+        got = got.float().cpu()
+        bound = 1e-4 + sharp * (1e-2 * want.abs().max() + RTOL[dtype] * want.abs())
+        ratio = ((got - want).abs() / bound).max().item()
+        assert ratio <= 0.5, f"{name} {tag}: {ratio:.2f} of the ordinary bar with delta from the rounded out"
+        bound_plain = 1e-4 + sharp * (1e-2 * want_plain.abs().max() + RTOL[dtype] * want_plain.abs())
+        worst_plain = max(worst_plain, ((got - want_plain).abs() / bound_plain).max().item())
+    print(f"  against the delta-free form: {worst_plain:.2f} of the ordinary bar", flush=True)
 
 
 @pytest.mark.parametrize("seed", range(40))
