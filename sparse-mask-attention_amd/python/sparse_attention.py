@@ -303,14 +303,14 @@ def pack_mask(mask: torch.Tensor) -> torch.Tensor:
     return sparse_attn_cuda.pack_mask(mask)
 
 
-def tile_map(mask_packed: torch.Tensor, min_skip: float = 0.25):
+def tile_map(mask_packed: torch.Tensor, min_skip: float = 0.3):
     """Occupancy of the 64 x 64 blocks of a packed mask, for ``sparse_attention(..., mask_packed=,
     tile_map=)``: int32 ``[B, H, T, 2, ceil(T/32)]`` with T = ceil(N/64); per block of 64 query rows
     one bit per 64-key tile "some entry kept", then one bit per tile "every entry kept".
 
     Returns None when the map would not pay: the forward walks the key tiles per 128 query rows (two
-    row blocks), and below ``min_skip`` (default a quarter) of those visits saved the walk costs what
-    it saves (a causal mask at N = 256 skips 6 of 32 visits per head and runs no faster with the
+    row blocks), and below ``min_skip`` (default 0.3) of those visits saved the walk costs what
+    it saves (a causal mask at N = 256 skips 2 of 8 visits per head and runs no faster with the
     map).  ``min_skip=0`` returns the map whenever a single visit disappears.  Synchronises with the
     device once, to look at that; meant to be called once for a mask that is used many times."""
     _require_ext(mask_packed)
