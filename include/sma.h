@@ -224,7 +224,8 @@ int sma_attn_fwd_map_strided(const sma_tensor *q, const sma_tensor *k, const sma
  * boolean bytes themselves and forms the packed words of each 64-key tile on the fly, so the packing
  * pass, its launch and the round trip of the words through memory disappear.
  *
- *   q, k, v, out    contiguous [B,H,N,D], D = 32, 64 or 128; 16 <= N <= 46340
+ *   q, k, v, out    contiguous [B,H,N,D] (sma_attn_fwd_bool_mask_strided takes strided ones), D = 32, 64
+ *                   or 128; 16 <= N <= 46340
  *   mask            uint8 [Bm,Hm,N,N] with Bm in {1,B}, Hm in {1,H}, rows contiguous, at any byte
  *                   address; a byte counts as "attend" when it is non-zero, as in sma_pack_mask;
  *                   mask_stride_b / mask_stride_h in BYTES, 0 = shared between batch entries /
@@ -261,6 +262,19 @@ int sma_attn_fwd_bool_mask_map(const void *q, const void *k, const void *v, cons
                                int64_t mask_stride_b, int64_t mask_stride_h, void *out, float *lse,
                                uint32_t *packed_out, uint32_t *map_out, int B, int H, int N, int D,
                                float scale, int dtype, void *stream);
+
+/* sma_attn_fwd_bool_mask_map for strided q, k, v, out (see sma_attn_fwd_strided for what a layout
+ * may be): a [B,N,H,D] buffer viewed as [B,H,N,D] or the slices of a fused qkv projection go through
+ * the one launch as they are.  The mask, lse, packed_out and map_out are as in
+ * sma_attn_fwd_bool_mask_map, which is this function with contiguous strides.
+ *
+ * Replaces: as sma_attn_fwd_bool_mask; the strides are those of SparseAttentionParams
+ *           (csrc/sparse_attention.h:30-33), which the reference declares and never reads.
+ */
+int sma_attn_fwd_bool_mask_strided(const sma_tensor *q, const sma_tensor *k, const sma_tensor *v,
+                                   const uint8_t *mask, int64_t mask_stride_b, int64_t mask_stride_h,
+                                   const sma_tensor *out, float *lse, uint32_t *packed_out, uint32_t *map_out,
+                                   int B, int H, int N, int D, float scale, int dtype, void *stream);
 
 /* sma_attn_bwd for strided dout, q, k, v, out, dq, dk, dv and a shared mask (see
  * sma_attn_fwd_strided); lse and delta_ws are contiguous float [B,H,N].

@@ -781,20 +781,27 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     default: kernel = attn_fwd_kernel<true, true, true, HDIM>; break;                  \
     }
 #define SMA_FWD_BYTEMASK_VARIANTS(HDIM)                                                 \
-    switch ((variant >> 1) | (byproducts ? 4 : 0)) {                                   \
-    case 0: kernel = attn_fwd_kernel<false, false, true, HDIM, true>; break;           \
-    case 1: kernel = attn_fwd_kernel<false, true, true, HDIM, true>; break;            \
-    case 2: kernel = attn_fwd_kernel<true, false, true, HDIM, true>; break;            \
-    case 3: kernel = attn_fwd_kernel<true, true, true, HDIM, true>; break;             \
-    case 4: kernel = attn_fwd_kernel<false, false, true, HDIM, true, true>; break;     \
-    case 5: kernel = attn_fwd_kernel<false, true, true, HDIM, true, true>; break;      \
-    case 6: kernel = attn_fwd_kernel<true, false, true, HDIM, true, true>; break;      \
+    switch (variant | (byproducts ? 8 : 0)) {                                          \
+    case 0: kernel = attn_fwd_kernel<false, false, false, HDIM, true>; break;          \
+    case 1: kernel = attn_fwd_kernel<false, false, true, HDIM, true>; break;           \
+    case 2: kernel = attn_fwd_kernel<false, true, false, HDIM, true>; break;           \
+    case 3: kernel = attn_fwd_kernel<false, true, true, HDIM, true>; break;            \
+    case 4: kernel = attn_fwd_kernel<true, false, false, HDIM, true>; break;           \
+    case 5: kernel = attn_fwd_kernel<true, false, true, HDIM, true>; break;            \
+    case 6: kernel = attn_fwd_kernel<true, true, false, HDIM, true>; break;            \
+    case 7: kernel = attn_fwd_kernel<true, true, true, HDIM, true>; break;             \
+    case 8: kernel = attn_fwd_kernel<false, false, false, HDIM, true, true>; break;    \
+    case 9: kernel = attn_fwd_kernel<false, false, true, HDIM, true, true>; break;     \
+    case 10: kernel = attn_fwd_kernel<false, true, false, HDIM, true, true>; break;    \
+    case 11: kernel = attn_fwd_kernel<false, true, true, HDIM, true, true>; break;     \
+    case 12: kernel = attn_fwd_kernel<true, false, false, HDIM, true, true>; break;    \
+    case 13: kernel = attn_fwd_kernel<true, false, true, HDIM, true, true>; break;     \
+    case 14: kernel = attn_fwd_kernel<true, true, false, HDIM, true, true>; break;     \
     default: kernel = attn_fwd_kernel<true, true, true, HDIM, true, true>; break;      \
     }
     const bool byproducts = a.mask_out != nullptr || a.map_out != nullptr;
     if (a.byte_mask) {
-        // built for contiguous rows only (checked by the C-ABI layer)
-        if (!packed || a.N < 16) return hipErrorInvalidValue;
+        if (a.N < 16) return hipErrorInvalidValue;          // a row holds at least one 16-byte copy (checked by the C-ABI layer)
         if (D == 32) { SMA_FWD_BYTEMASK_VARIANTS(32) } else if (D == 64) { SMA_FWD_BYTEMASK_VARIANTS(64) } else { SMA_FWD_BYTEMASK_VARIANTS(128) }
     } else if (D == 32) { SMA_FWD_VARIANTS(32) } else if (D == 64) { SMA_FWD_VARIANTS(64) } else { SMA_FWD_VARIANTS(128) }
 #undef SMA_FWD_VARIANTS

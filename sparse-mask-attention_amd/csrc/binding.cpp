@@ -127,15 +127,22 @@ void forward(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor
 }
 
 // Limits of sma_attn_fwd_bool_mask, so that callers can choose between it and pack_mask + forward
-// without provoking an error: contiguous q, k, v, head dim 32, 64 or 128, 16 <= N < 46341, a
-// contiguous bool mask [1|B, 1|H, N, N].
+// without provoking an error: q, k, v with contiguous rows and strides that are multiples of 8
+// elements, head dim 32, 64 or 128, 16 <= N < 46341, a contiguous bool mask [1|B, 1|H, N, N].
 bool bool_mask_supported(const torch::Tensor &q, const torch::Tensor &k, const torch::Tensor &v,
                          const torch::Tensor &mask)
 {
     if (!q.is_cuda() || q.dim() != 4 || mask.dim() != 4) return false;
     const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
     if (!(D == 32 || D == 64 || D == 128) || N < 16 || N * N >= (int64_t(1) << 31)) return false;
-    if (!q.is_contiguous() || !k.is_contiguous() || !v.is_contiguous()) return false;
+    // q, k, v as the strided entry points take them: rows contiguous, other strides multiples of 8
+    // elements, 16-byte aligned storage
+    for (const torch::Tensor *t : {&q, &k, &v}) {
+        if (t->dim() != 4 || t->sizes() != q.sizes() || (t->stride(3) != 1 && t->size(3) != 1)) return false;
+        if (reinterpret_cast<uintptr_t>(t->data_ptr()) % 16 != 0) return false;
+        for (int d = 0; d < 3; ++d)
+            if (t->size(d) > 1 && (t->stride(d) < 0 || t->stride(d) % 8 != 0)) return false;
+    }
     if (mask.scalar_type() != at::kBool || !mask.is_contiguous() || mask.device() != q.device()) return false;
     if (!((mask.size(0) == B || mask.size(0) == 1) && (mask.size(1) == H || mask.size(1) == 1) &&
           mask.size(2) == N && mask.size(3) == N))
@@ -157,15 +164,15 @@ void forward_bool_mask(const torch::Tensor &q, const torch::Tensor &k, const tor
     const auto dt = q.scalar_type();
     TORCH_CHECK(dt == at::kHalf || dt == at::kBFloat16, "Unsupported dtype, need BF16 or FP16");
     TORCH_CHECK(bool_mask_supported(q, k, v, mask),
-                "forward_bool_mask needs contiguous q, k, v with head_dim 32, 64 or 128, N >= 16 and a "
-                "contiguous bool mask [B or 1, H or 1, N, N]; use pack_mask + forward otherwise");
+                "forward_bool_mask needs q, k, v with contiguous rows (strides multiples of 8 elements), head_dim "
+                "32, 64 or 128, N >= 16 and a contiguous bool mask [B or 1, H or 1, N, N]; use pack_mask + forward otherwise");
     const int64_t B = q.size(0), H = q.size(1), N = q.size(2), D = q.size(3);
     for (const torch::Tensor *t : {&k, &v, static_cast<const torch::Tensor *>(&out)}) {
         TORCH_CHECK(t->device() == q.device(), "q, k, v, out must be on the same device");
         TORCH_CHECK(t->scalar_type() == dt, "q, k, v, out must have the same dtype");
         TORCH_CHECK(t->sizes() == q.sizes(), "q, k, v, out must have the same shape");
     }
-    TORCH_CHECK(out.is_contiguous(), "out must be contiguous");
+    const sma_tensor tq = rows_of(q, "q"), tk = rows_of(k, "k"), tv = rows_of(v, "v"), to = rows_of(out, "out");
     float *lse_ptr = nullptr;
     if (is_training) {
         TORCH_CHECK(lse.has_value() && lse->defined(), "is_training=True needs an lse tensor");
@@ -199,12 +206,12 @@ void forward_bool_mask(const torch::Tensor &q, const torch::Tensor &k, const tor
     const int64_t msh = mask.size(1) == 1 ? 0 : N * N;
     const c10::DeviceGuard guard(q.device());
     hipStream_t stream = c10::hip::getCurrentHIPStream(q.device().index()).stream();
-    const int st = sma_attn_fwd_bool_mask_map(q.data_ptr(), k.data_ptr(), v.data_ptr(),
-                                              reinterpret_cast<const uint8_t *>(mask.data_ptr<bool>()), msb, msh,
-                                              out.data_ptr(), lse_ptr, packed_ptr, map_ptr, (int)B, (int)H, (int)N,
-                                              (int)D, (float)scale,
-                                              dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
-    check_status(st, "sma_attn_fwd_bool_mask_map");
+    const int st = sma_attn_fwd_bool_mask_strided(&tq, &tk, &tv,
+                                                  reinterpret_cast<const uint8_t *>(mask.data_ptr<bool>()), msb, msh,
+                                                  &to, lse_ptr, packed_ptr, map_ptr, (int)B, (int)H, (int)N,
+                                                  (int)D, (float)scale,
+                                                  dt == at::kBFloat16 ? SMA_DTYPE_BF16 : SMA_DTYPE_F16, stream);
+    check_status(st, "sma_attn_fwd_bool_mask_strided");
 }
 
 // backward(dout, q, k, v, out, lse, mask_packed, dq, dk, dv, scale) -> None, the call the

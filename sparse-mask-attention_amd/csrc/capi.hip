@@ -312,6 +312,16 @@ int sma_attn_fwd_bool_mask_map(const void *q, const void *k, const void *v, cons
                                uint32_t *packed_out, uint32_t *map_out, int B, int H, int N, int D,
                                float scale, int dtype, void *stream)
 {
+    const sma_tensor t[4] = {dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D), dense(out, H, N, D)};
+    return sma_attn_fwd_bool_mask_strided(&t[0], &t[1], &t[2], mask, mask_stride_b, mask_stride_h, &t[3], lse,
+                                          packed_out, map_out, B, H, N, D, scale, dtype, stream);
+}
+
+int sma_attn_fwd_bool_mask_strided(const sma_tensor *q, const sma_tensor *k, const sma_tensor *v,
+                                   const uint8_t *mask, int64_t mask_stride_b, int64_t mask_stride_h,
+                                   const sma_tensor *out, float *lse, uint32_t *packed_out, uint32_t *map_out,
+                                   int B, int H, int N, int D, float scale, int dtype, void *stream)
+{
     if (B < 0 || H < 0 || N < 0 || D < 0) return SMA_ERR_BAD_SHAPE;
     if (D != 32 && D != 64 && D != 128) return SMA_ERR_HEAD_DIM;
     if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
@@ -330,16 +340,16 @@ int sma_attn_fwd_bool_mask_map(const void *q, const void *k, const void *v, cons
     // N * N above is the tighter one)
     if (map_out && (N + 63) / 64 > 32 * 32) return SMA_ERR_BAD_SHAPE;
     if (mask_stride_b < 0 || mask_stride_h < 0) return SMA_ERR_STRIDE;
-    // mask rows start at any byte address: the kernel's 16-byte copies rely on the device serving them
-    if (sma::unaligned_access_state(static_cast<hipStream_t>(stream)) == 0) return SMA_ERR_DEVICE;
 
     sma::AttnArgs a;
-    const sma_tensor t[4] = {dense(q, H, N, D), dense(k, H, N, D), dense(v, H, N, D), dense(out, H, N, D)};
+    const sma_tensor *in[4] = {q, k, v, out};
     sma::Rows *to[4] = {&a.q, &a.k, &a.v, &a.out};
     for (int i = 0; i < 4; ++i) {
-        const int st = to_rows(&t[i], B, H, N, D, i == 3, to[i]);
+        const int st = to_rows(in[i], B, H, N, D, i == 3, to[i]);
         if (st != SMA_OK) return st;
     }
+    // mask rows start at any byte address: the kernel's 16-byte copies rely on the device serving them
+    if (sma::unaligned_access_state(static_cast<hipStream_t>(stream)) == 0) return SMA_ERR_DEVICE;
     a.mask = sma::PackedMask{reinterpret_cast<const uint32_t *>(mask), mask_stride_b, mask_stride_h};
     a.lse = lse;
     a.BH = (int)BH;

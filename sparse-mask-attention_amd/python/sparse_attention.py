@@ -32,7 +32,7 @@ What differs from the reference, on purpose:
 * Head dims: the kernels exist for 64 (the reference's only one), 32 and 128.  Any other D <= 128
   is computed exactly by zero-padding q, k, v to the next of these (the scores and the first D output
   columns do not change; the scale stays 1/sqrt(D)) at the price of the padding copies.
-* The mask is not packed in a pass of its own: where the kernel's limits allow (contiguous q, k, v,
+* The mask is not packed in a pass of its own: where the kernel's limits allow (any q, k, v the strided kernels take,
   N >= 16) one launch reads the bool mask itself and forms the packed words tile by
   tile, which is 15-35 % faster than pack + attention; under autograd the same launch also leaves
   the packed words behind for the backward.  Otherwise the mask is packed as the reference does.

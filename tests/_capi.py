@@ -81,6 +81,8 @@ def load():
         lib.sma_attn_fwd_bool_mask.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         lib.sma_attn_fwd_bool_mask_map.restype = ci
         lib.sma_attn_fwd_bool_mask_map.argtypes = [vp, vp, vp, vp, i64, i64, vp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
+        lib.sma_attn_fwd_bool_mask_strided.restype = ci
+        lib.sma_attn_fwd_bool_mask_strided.argtypes = [tp, tp, tp, vp, i64, i64, tp, vp, vp, vp, ci, ci, ci, ci, cf, ci, vp]
         _lib = lib
     return _lib
 
@@ -270,6 +272,38 @@ def attn_fwd_strided(q, k, v, packed, out=None, scale=None, want_lse=False):
                                   lse.data_ptr() if want_lse else None, B, H, N, D, scale, dt, _stream())
     assert st == SMA_OK, lib.sma_strerror(st)
     return (out, lse) if want_lse else out
+
+
+def attn_fwd_bool_mask_strided(q, k, v, mask, out=None, scale=None, want_lse=False, want_packed=False, want_map=False,
+                               expect=SMA_OK):
+    """Forward straight from the boolean mask through sma_attn_fwd_bool_mask_strided: q, k, v (and out,
+    if given) may be any views whose last dimension is contiguous.  Returns out (and lse) (and the
+    packed words) (and the tile map), or the status if `expect` is an error code."""
+    lib = load()
+    B, H, N, D = q.shape
+    if scale is None:
+        scale = 1.0 / (D ** 0.5)
+    dt = {torch.float16: SMA_DTYPE_F16, torch.bfloat16: SMA_DTYPE_BF16}[q.dtype]
+    assert mask.dtype == torch.bool and mask.is_contiguous()
+    Bm, Hm = mask.shape[:2]
+    msb = Hm * N * N if Bm == B and B > 1 else 0
+    msh = N * N if Hm == H and H > 1 else 0
+    if out is None:
+        out = torch.full((B, H, N, D), float("nan"), dtype=q.dtype, device=q.device)
+    lse = torch.full((B, H, N), float("nan"), dtype=torch.float32, device=q.device) if want_lse else None
+    packed = (torch.full((Bm, Hm, N, (N + 31) // 32), -1431655766, dtype=torch.int32, device=q.device)
+              if want_packed else None)
+    tm = _new_map(Bm, Hm, N, q.device) if want_map else None
+    tq, tk, tv, to = (SmaTensor.of(t) for t in (q, k, v, out))
+    st = lib.sma_attn_fwd_bool_mask_strided(tq, tk, tv, mask.data_ptr(), msb, msh, to,
+                                            lse.data_ptr() if want_lse else None,
+                                            packed.data_ptr() if want_packed else None,
+                                            tm.data_ptr() if want_map else None, B, H, N, D, scale, dt, _stream())
+    if expect != SMA_OK:
+        return st
+    assert st == SMA_OK, lib.sma_strerror(st)
+    res = (out,) + ((lse,) if want_lse else ()) + ((packed,) if want_packed else ()) + ((tm,) if want_map else ())
+    return res if len(res) > 1 else out
 
 
 def attn_bwd_strided(dout, q, k, v, out, lse, packed, grads=None, scale=None):

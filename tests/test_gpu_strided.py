@@ -1,4 +1,5 @@
-"""GPU parity of the strided entry points (sma_attn_fwd_strided / sma_attn_bwd_strided): tensors
+"""GPU parity of the strided entry points (sma_attn_fwd_strided / sma_attn_bwd_strided /
+sma_attn_fwd_bool_mask_strided): tensors
 that are views with explicit strides, and packed masks shared between batch entries and heads.
 
 The reference reserves strides in its parameter block (csrc/sparse_attention.h:30-33) without ever
@@ -59,6 +60,63 @@ def test_forward_on_slices_of_a_fused_qkv_buffer(dev):
     torch.cuda.synchronize()
     assert torch.equal(got, want)
     assert (store[..., 64:] == 7.0).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [32, 64, 128])
+@pytest.mark.parametrize("N", [16, 100, 257, 512])
+def test_forward_from_the_bool_mask_on_strided_views_equals_dense(dev, dtype, D, N):
+    """The one launch that reads the boolean mask, on a [B,N,H,D] buffer viewed as [B,H,N,D] and on
+    slices of a fused qkv buffer with padded output rows: bit for bit what the dense entry point gives
+    on contiguous copies (output, lse, the packed words and the tile map it leaves behind), gaps
+    between rows untouched."""
+    B, H = 2, 3
+    g = torch.Generator().manual_seed(1000 * D + N)
+    q, k, v = (torch.randn(B, H, N, D, generator=g).to(dtype) for _ in range(3))
+    mask = torch.rand(B, H, N, N, generator=g) < 0.3
+    mask[:, :, :, N // 2:] &= torch.rand(B, H, 1, 1, generator=g) < 0.5          # some heads keep half the keys only
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    want, want_lse, want_packed, want_map = _capi.attn_fwd_bool_mask(qd, kd, vd, md, want_lse=True, want_packed=True,
+                                                                     want_map=True)
+    # [B, N, H, D] views, output stored [B, N, H, D] too
+    qs, ks, vs = (_bnhd(t) for t in (qd, kd, vd))
+    out_store = torch.full((B, N, H, D), float("nan"), dtype=dtype, device=dev)
+    got, lse, packed, tm = _capi.attn_fwd_bool_mask_strided(qs, ks, vs, md, out=out_store.permute(0, 2, 1, 3),
+                                                            want_lse=True, want_packed=True, want_map=True)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and torch.equal(lse, want_lse)
+    assert torch.equal(packed, want_packed) and torch.equal(tm, want_map)
+    # slices of one [B, N, 3, H, D] buffer, output rows padded by 32 elements
+    qkv = torch.stack([qd, kd, vd], dim=0).permute(1, 3, 0, 2, 4).contiguous()
+    qs, ks, vs = (qkv[:, :, i].permute(0, 2, 1, 3) for i in range(3))
+    store = torch.full((B, H, N, D + 32), 7.0, dtype=dtype, device=dev)
+    got = _capi.attn_fwd_bool_mask_strided(qs, ks, vs, md, out=store[..., :D])
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and (store[..., D:] == 7.0).all()
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    assert torch.allclose(got.float().cpu(), ref, atol=1e-2, rtol=2e-2)
+
+
+def test_python_api_takes_strided_views_through_the_one_launch_path(dev):
+    """sparse_attention_func / sparse_attention on [B,N,H,D] views: the module says the one-launch
+    forward applies, and results (and gradients) are those of contiguous copies, bit for bit."""
+    import importlib
+    sa = importlib.import_module("python.sparse_attention")
+    B, H, N = 2, 4, 200
+    g = torch.Generator().manual_seed(77)
+    q, k, v, do = (torch.randn(B, N, H, 64, generator=g).half().to(dev).permute(0, 2, 1, 3) for _ in range(4))
+    mask = (torch.rand(B, H, N, N, generator=g) < 0.3).to(dev)
+    assert not q.is_contiguous() and sa.sparse_attn_cuda.bool_mask_supported(q, k, v, mask)
+    want = sa.sparse_attention_func(q.contiguous(), k.contiguous(), v.contiguous(), mask)
+    assert torch.equal(sa.sparse_attention_func(q, k, v, mask), want)
+    grads = []
+    for conv in (lambda t: t, lambda t: t.contiguous()):
+        leaves = [conv(t).clone().requires_grad_(True) for t in (q, k, v)]
+        out = sa.sparse_attention(*leaves, mask)
+        out.backward(conv(do))
+        grads.append([out.detach()] + [t.grad for t in leaves])
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
 
 
 @pytest.mark.parametrize("shape", ["11", "B1", "1H"])
