@@ -63,6 +63,17 @@ def event_time_ms(fn, warmup, repeat, torch):
     return start.elapsed_time(end) / repeat
 
 
+def settle(fn, torch, ms=60.0):
+    """Run fn back to back for `ms` milliseconds, untimed: after the host-side pauses between the
+    sections of this script (building tensors on the CPU, copies) the device needs tens of
+    milliseconds of work to be back at the clock it keeps under load."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < ms * 1e-3:
+        for _ in range(20):
+            fn()
+        torch.cuda.synchronize()
+
+
 def cold_time_ms(make_call, n_sets, warmup, repeat, torch):
     """Mean ms per call when consecutive calls use different copies of every tensor: make_call(i)
     returns the call for copy i, n_sets copies exceed the caches, so no call finds its inputs (or
@@ -205,6 +216,11 @@ def main():
             "bwd": lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale),
             "bwd_map": lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale, full_map),
         }[args.only]
+        t_pre = time.perf_counter()          # to the device's steady clock first, as for the whole line
+        while time.perf_counter() - t_pre < args.precondition_ms * 1e-3:
+            for _ in range(50):
+                fn()
+            torch.cuda.synchronize()
         ms = event_time_ms(fn, args.warmup, args.steps, torch)
         print(json.dumps({"only": args.only, "workload": w.name, "launches": args.steps, "ms": round(ms, 5)}), flush=True)
         return
@@ -274,6 +290,7 @@ def main():
     # clock the part has settled at, what the caches hold) moves a single measurement by several
     # per cent, and differences between these kernels are read off this line.
     timings = {name: [] for name in kernels}
+    settle(kernels["attn"], torch)
     for rnd in range(3):
         for name, fn in kernels.items():
             timings[name].append(event_time_ms(fn, 10, reps, torch))
@@ -287,8 +304,9 @@ def main():
     ext.forward(qd, kd, vd, packed, out, lse, scale, True)
     dout = torch.randn(qd.shape, generator=torch.Generator().manual_seed(43)).to(qd.dtype).to(dev)
     dq, dk, dv = (torch.empty_like(qd) for _ in range(3))
-    bwd_ms = event_time_ms(lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale, tmap),
-                           5, reps, torch)
+    bwd_call = lambda: ext.backward(dout, qd, kd, vd, out, lse, packed, dq, dk, dv, scale, tmap)
+    settle(bwd_call, torch)
+    bwd_ms = sorted(event_time_ms(bwd_call, 5, reps, torch) for _ in range(3))[1]
     bwd_tflops = w.bwd_dense_flops / (bwd_ms * 1e-3) / 1e12
 
     # ---- the same kernels with nothing cached: rotate through copies of every tensor (> 512 MB) ----
@@ -296,6 +314,7 @@ def main():
     n_sets = max(3, -(-(640 << 20) // set_bytes))
     copies = [(qd.clone(), kd.clone(), vd.clone(), md.clone(), packed.clone(), torch.empty_like(qd))
               for _ in range(n_sets)]
+    settle(kernels["attn"], torch)
     attn_cold_ms = cold_time_ms(lambda i: (lambda c=copies[i]: ext.forward(c[0], c[1], c[2], c[4], c[5], None, scale,
                                                                             False, tmap)), n_sets, 10, reps, torch)
     pack_cold_ms = cold_time_ms(lambda i: (lambda c=copies[i]: lib.sma_pack_mask(c[3].data_ptr(), c[4].data_ptr(),
