@@ -167,6 +167,10 @@ def main():
                          "the same leaving lse, packed words and tile map behind, pack = the packer, bwd / "
                          "bwd_map = the backward without / with the tile map.  For rocprofv3 runs whose "
                          "per-kernel averages must not blend launch contexts.")
+    ap.add_argument("--ramp", action="store_true",
+                    help="instead of the benchmark: time the step in consecutive blocks from the first launch after "
+                         "idling (10 blocks of 20 steps, then 50 of 200) and print one line per block; shows the "
+                         "clock ramp that --precondition-ms skips")
     ap.add_argument("--calib-copy-mib", type=int, default=0,
                     help="also run one plain device-to-device copy of this many MiB (a traffic yardstick "
                          "for rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs)")
@@ -249,6 +253,22 @@ def main():
             fn()
         torch.cuda.synchronize()
         return (time.perf_counter() - t0) * 1e3 / args.steps
+
+    if args.ramp:
+        torch.cuda.synchronize()
+        time.sleep(0.5)                      # idle first
+        t00 = time.perf_counter()
+        for blk in range(60):
+            n = 20 if blk < 10 else 200
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for _ in range(n):
+                step()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            print(json.dumps({"block": blk, "steps": n, "starts_at_ms": round((t0 - t00) * 1e3, 2),
+                              "us_per_step": round((t1 - t0) * 1e6 / n, 2)}), flush=True)
+        return
 
     # Before anything is timed the device is brought to its steady clock: for the first 25-30 ms of
     # work after idling the part runs this step 5 to 25 % slower than it then settles at (measured:
