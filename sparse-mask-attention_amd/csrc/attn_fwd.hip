@@ -532,6 +532,14 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         if (__builtin_amdgcn_ballot_w64((w2.x | w2.y) != 0u) == 0ull) return;
         // ---- S^T: sacc[blk][4g+j] = log2 weight / pm of (key 32blk + 8g + 4hh + j, query l32) ----
         f32x16 sacc[2];
+        // The K fragments of MFMA step s + 1 are requested before the MFMAs of step s are issued, the
+        // first pair before the table look-ups below.  The scheduling barriers hold that order: left
+        // alone, the compiler requests each pair just before its MFMAs (it saves eight registers)
+        // and the wavefront sits out four LDS round trips per tile one after the other.
+        u32x4 kf[2][2];
+        kf[0][0] = lds_read_b128(kaddr[0] + so);
+        kf[0][1] = lds_read_b128(kaddr[0] + so + 4096);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int blk = 0; blk < 2; ++blk) {
             const uint32_t wa = (blk == 0 ? w2.x : w2.y) << nib_shift;
@@ -548,9 +556,15 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         }
 #pragma unroll
         for (int s = 0; s < KS; ++s) {
-            const uint32_t ka = kaddr[s & 3] + so + (s >> 2) * TILE_BYTES;
-            sacc[0] = E::mfma(lds_read_b128(ka), qf[s], sacc[0]);
-            sacc[1] = E::mfma(lds_read_b128(ka + 4096), qf[s], sacc[1]);
+            if (s + 1 < KS) {
+                const uint32_t ka = kaddr[(s + 1) & 3] + so + ((s + 1) >> 2) * TILE_BYTES;
+                kf[(s + 1) & 1][0] = lds_read_b128(ka);
+                kf[(s + 1) & 1][1] = lds_read_b128(ka + 4096);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+            sacc[0] = E::mfma(kf[s & 1][0], qf[s], sacc[0]);
+            sacc[1] = E::mfma(kf[s & 1][1], qf[s], sacc[1]);
+            __builtin_amdgcn_sched_barrier(0);
         }
         // ---- the row maximum of the tile is taken only when it can matter ----
         // Moves the reference point when a row's scores leave the window [r-8, r+8] upwards, or when
