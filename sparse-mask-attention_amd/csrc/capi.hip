@@ -10,6 +10,14 @@ namespace {
 
 inline bool misaligned(const void *p, uintptr_t a) { return (reinterpret_cast<uintptr_t>(p) & (a - 1)) != 0; }
 
+// a * b < 2^31 for non-negative a, b, without forming a product that could overflow 64 bits
+// (B * H alone may reach 2^62)
+inline bool below_2_31(long long a, long long b)
+{
+    const long long lim = 1ll << 31;
+    return a == 0 || b == 0 || (a < lim && b < lim && a * b < lim);
+}
+
 inline sma_tensor dense(const void *p, int H, int N, int D)
 {
     return sma_tensor{const_cast<void *>(p), (int64_t)H * N * D, (int64_t)N * D, (int64_t)D};
@@ -96,7 +104,7 @@ int sma_tile_map(const uint32_t *mask_packed, uint32_t *tile_map, int B, int H, 
     if (slabs == 0 || N == 0) return SMA_OK;
     if (mask_packed == nullptr || tile_map == nullptr) return SMA_ERR_NULL_POINTER;
     if (misaligned(mask_packed, 4) || misaligned(tile_map, 4)) return SMA_ERR_ALIGNMENT;
-    if (slabs * ((N + 63) / 64) >= (1ll << 31) || N > 131072) return SMA_ERR_BAD_SHAPE;
+    if (N > 131072 || !below_2_31(slabs, (N + 63) / 64)) return SMA_ERR_BAD_SHAPE;
     const hipError_t e = sma::launch_tile_map(mask_packed, tile_map, slabs, N, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
 }
@@ -111,7 +119,7 @@ int sma_pack_mask_map(const uint8_t *mask, uint32_t *packed, uint32_t *tile_map,
 {
     // what sma_tile_map would refuse is refused before anything is written
     if (tile_map != nullptr && B >= 0 && H >= 0 &&
-        (N > 131072 || (long long)B * H * ((N + 63) / 64) >= (1ll << 31) || misaligned(tile_map, 4)))
+        (N > 131072 || !below_2_31((long long)B * H, (N + 63) / 64) || misaligned(tile_map, 4)))
         return misaligned(tile_map, 4) ? SMA_ERR_ALIGNMENT : SMA_ERR_BAD_SHAPE;
     const int st = sma_pack_mask(mask, packed, B, H, N, stream);
     if (st != SMA_OK || tile_map == nullptr) return st;
@@ -121,11 +129,11 @@ int sma_pack_mask_map(const uint8_t *mask, uint32_t *packed, uint32_t *tile_map,
 int sma_pack_mask(const uint8_t *mask, uint32_t *packed, int B, int H, int N, void *stream)
 {
     if (B < 0 || H < 0 || N < 0) return SMA_ERR_BAD_SHAPE;
-    const long long rows = (long long)B * H * N;
-    if (rows == 0) return SMA_OK;
+    if (B == 0 || H == 0 || N == 0) return SMA_OK;
     if (mask == nullptr || packed == nullptr) return SMA_ERR_NULL_POINTER;
     const long long nw = (N + 31) / 32;
-    if (rows * nw >= (1ll << 31) || rows >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
+    if (!below_2_31((long long)B * H, N) || !below_2_31((long long)B * H * N, nw)) return SMA_ERR_BAD_SHAPE;
+    const long long rows = (long long)B * H * N;
     if (misaligned(packed, 4)) return SMA_ERR_ALIGNMENT;
     const hipError_t e = sma::launch_pack_mask(mask, packed, rows, N, static_cast<hipStream_t>(stream));
     return e == hipSuccess ? SMA_OK : SMA_ERR_LAUNCH;
@@ -172,7 +180,7 @@ int sma_attn_bwd_map_strided(const sma_tensor *dout, const sma_tensor *q, const 
     if (BH == 0 || N == 0) return SMA_OK;
     if (!lse || !mask_packed || !delta_ws) return SMA_ERR_NULL_POINTER;
     const long long qtiles = (N + 127) / 128;
-    if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
+    if (!below_2_31(BH, qtiles) || !below_2_31(BH, N)) return SMA_ERR_BAD_SHAPE;
     // a lane's byte offset into the packed mask of one (b,h) is a 32-bit register
     if ((long long)N * ((N + 31) / 32) * 4 >= (1ll << 32)) return SMA_ERR_BAD_SHAPE;
     if (misaligned(mask_packed, 4) || misaligned(lse, 4) || misaligned(delta_ws, 4) || (tile_map && misaligned(tile_map, 4)))
@@ -242,7 +250,7 @@ int sma_attn_fwd_map_strided(const sma_tensor *q, const sma_tensor *k, const sma
     if (BH == 0 || N == 0) return SMA_OK;
     if (!mask_packed) return SMA_ERR_NULL_POINTER;
     const long long qtiles = (N + 127) / 128;
-    if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
+    if (!below_2_31(BH, qtiles) || !below_2_31(BH, N)) return SMA_ERR_BAD_SHAPE;
     // a lane's byte offset into the packed mask of one (b,h) is a 32-bit register
     if ((long long)N * ((N + 31) / 32) * 4 >= (1ll << 32)) return SMA_ERR_BAD_SHAPE;
     if (misaligned(mask_packed, 4) || (lse && misaligned(lse, 4)) || (tile_map && misaligned(tile_map, 4)))
@@ -331,7 +339,7 @@ int sma_attn_fwd_bool_mask_strided(const sma_tensor *q, const sma_tensor *k, con
     if (!mask) return SMA_ERR_NULL_POINTER;
     if (N < 16) return SMA_ERR_BAD_SHAPE;               // a row holds at least one 16-byte copy
     const long long qtiles = (N + 127) / 128;
-    if (BH * qtiles >= (1ll << 31) || BH * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
+    if (!below_2_31(BH, qtiles) || !below_2_31(BH, N)) return SMA_ERR_BAD_SHAPE;
     // a lane's byte offset into the mask of one (b,h) is a 32-bit register
     if ((long long)N * N >= (1ll << 31)) return SMA_ERR_BAD_SHAPE;
     if ((lse && misaligned(lse, 4)) || (packed_out && misaligned(packed_out, 4)) || (map_out && misaligned(map_out, 4)))
@@ -391,7 +399,7 @@ int sma_attn_bwd_static_ws(const void *dout, const void *q, const void *k, const
     if (dtype != SMA_DTYPE_F16 && dtype != SMA_DTYPE_BF16) return SMA_ERR_DTYPE;
     if (!isfinite(scale)) return SMA_ERR_SCALE;
     if (B == 0 || H == 0 || N == 0) return SMA_OK;
-    if ((long long)B * H > STATIC_WS_ROWS || (long long)B * H * (long long)N > STATIC_WS_ROWS) return SMA_ERR_WORKSPACE;
+    if ((long long)B * H > STATIC_WS_ROWS || (long long)B * H * N > STATIC_WS_ROWS) return SMA_ERR_WORKSPACE;
     float *ws = static_workspace();
     if (ws == nullptr) return SMA_ERR_LAUNCH;
     // Both kernels run on `stream`, the first writes every entry the second reads: nothing has to

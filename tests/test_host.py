@@ -125,6 +125,15 @@ def test_argument_validation_needs_no_gpu(capi):
     assert g(p, p, 0, 4, 8, None) == _capi.SMA_OK
     assert g(p, ctypes.c_void_p(0x1001), 1, 1, 8, None) == _capi.SMA_ERR_ALIGNMENT
 
+    # extents whose products pass 2^63 are refused like any other index range, by every entry point
+    huge = (1 << 31) - 1
+    assert g(p, p, huge, huge, huge, None) == _capi.SMA_ERR_BAD_SHAPE
+    assert capi.sma_tile_map(p, p, huge, huge, 64, None) == _capi.SMA_ERR_BAD_SHAPE
+    assert capi.sma_pack_mask_map(p, p, p, huge, huge, 64, None) == _capi.SMA_ERR_BAD_SHAPE
+    assert call(B=huge, H=huge, N=huge) == _capi.SMA_ERR_BAD_SHAPE
+    assert bcall(B=huge, H=huge, N=1024) == _capi.SMA_ERR_BAD_SHAPE
+    assert capi.sma_attn_bwd(*([p] * 11), huge, huge, 4096, 64, 0.125, 0, None) == _capi.SMA_ERR_BAD_SHAPE
+
 
 def test_python_api_surface_and_loud_failure_off_gpu():
     import python as pkg
