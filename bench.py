@@ -123,6 +123,20 @@ def source_digest(kernel):
     return h.hexdigest()[:16]
 
 
+def roofline_ceiling(flops, algorithmic_bytes, achieved_tflops):
+    """Where a kernel sits on the roofline: its FLOP per algorithmic byte against the machine's
+    balance (MFMA peak / HBM peak), the ceiling the model gives it (the lower of the MFMA peak and
+    FLOP-per-byte x HBM peak) and the fraction of that ceiling it reaches.  `frac` of the roofline
+    objects stays the fraction of the MFMA peak whichever side the kernel is on."""
+    import harness
+    balance = harness.MI355X_MFMA_F16_TFLOPS * 1e3 / harness.MI355X_HBM_GBPS
+    ai = flops / algorithmic_bytes
+    ceiling = min(harness.MI355X_MFMA_F16_TFLOPS, ai * harness.MI355X_HBM_GBPS / 1e3)
+    return {"flop_per_byte": round(ai, 1), "machine_balance_flop_per_byte": round(balance, 1),
+            "ceiling_side": "hbm" if ai < balance else "mfma", "ceiling_tflops": round(ceiling, 1),
+            "frac_of_ceiling": round(achieved_tflops / ceiling, 4)}
+
+
 def measured_traffic(workload, *kernels):
     """HBM bytes per launch (summed over `kernels`) from the committed rocprofv3 counter summaries
     of this workload (FETCH_SIZE and WRITE_SIZE, each scaled by what the same counter reads for a
@@ -414,6 +428,7 @@ def main():
                          "traffic": measured_traffic(w.name, "attn_bwd_dq_kernel", "attn_bwd_dkv_kernel"), "algorithmic_bytes": w.bwd_bytes},
     }
 
+    result["roofline_attn"].update(roofline_ceiling(w.dense_flops, w.attn_bytes, attn_tflops))
     if one_launch:
         gbps = w.fused_bytes / (fused_ms * 1e-3) / 1e9
         tfl = w.dense_flops / (fused_ms * 1e-3) / 1e12
@@ -435,6 +450,7 @@ def main():
                               "cache_note": "frac / hbm_frac: same tensors every launch, working set inside the 256 MB "
                                             "last-level cache (the reference's protocol); *_cold: rotating copies, "
                                             "every launch reads from HBM"}
+        result["roofline"].update(roofline_ceiling(w.dense_flops, w.fused_bytes, tfl))
     else:
         result["roofline"] = dict(result["roofline_attn"])
 
