@@ -67,9 +67,9 @@ def _draw(seed):
     return D, dtype, B, H, N, Bm, Hm, scale, layouts, q, k, v, do, mask
 
 
-# Seeds outside the 40 below on which dq misses the ordinary bar (found by drawing 59 360 more of
-# them once; all have N = 7, almost all are bf16): kept as a fixed list.
-FLOOR_SEEDS = [8315, 15725, 23526, 54200]
+# Seeds outside the 40 below on which dq misses the ordinary bar (found by drawing some 63 000 more of
+# them; all have N = 7, almost all are bf16): kept as a fixed list.
+FLOOR_SEEDS = [8315, 15725, 23526, 54200, 101365]
 
 
 @pytest.mark.parametrize("seed", FLOOR_SEEDS)
