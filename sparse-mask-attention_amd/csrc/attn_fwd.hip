@@ -429,7 +429,7 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
 
     // ================================ prologue: one memory round trip ================================
     // Requested at once, oldest first: q (this wave's 32 rows, staged through the second K/V stage,
-    // which the prologue leaves unused, K-swizzled), then the mask words and K/V of tile 0.
+    // which the prologue leaves unused, K-swizzled), then K/V and the mask words of tile 0.
     {
         const int qbase = qt * BM + wave * 32 < N ? qt * BM + wave * 32 : N - 1;   // wave-uniform
         const uint16_t *qsrc = qb + (size_t)qbase * q_sn;
@@ -469,8 +469,8 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     };
     const int t_first = next_tile();
     if (t_first < T) {
-        issue_mask(t_first, integral_constant<int, 0>{});
         issue_kv(t_first, integral_constant<int, 0>{});
+        issue_mask(t_first, integral_constant<int, 0>{});
     }
     // small LDS table for the mask: entry n (16 B) holds four floats, float j = (bit j of n) ? 0 : -inf
     if (tid < 64)
@@ -661,7 +661,7 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     // slot i % 2; the loop is unrolled by 2 so that these are constants.
     // In a visit of tile t:
     //   wait for the copies of tile t  ->  barrier  ->  request the copies of the next tile to be
-    //   visited (mask words, then K/V) into the stage the barrier has freed  ->  compute, unless
+    //   visited (K/V, then the mask words) into the stage the barrier has freed  ->  compute, unless
     //   this wave's 32 x 64 block of mask bits is empty.
     // (A ring of three stages, copies two tiles ahead, measured the same to 2 % slower on every
     // workload and costs 18 KB more LDS.)
@@ -682,9 +682,9 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         if (ragged && t == T - 1) zero_tail_rows(t, SLOT);
         __syncthreads();          // tile t landed for every wave; the stage of the previous visit is free
         const u32x2 w2 = mask_words(t, SLOT);
-        if (t_next < T) {
-            issue_mask(t_next, integral_constant<int, SLOT2>{});
+        if (t_next < T) {       // K/V first: the MFMA operands are what the next visit needs first (1-2 % with a byte mask)
             issue_kv(t_next, integral_constant<int, SLOT2>{});
+            issue_mask(t_next, integral_constant<int, SLOT2>{});
         }
         compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
     };
