@@ -106,9 +106,17 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_
 // BYPRODUCTS (with BYTEMASK): the caller wants the packed words and / or the tile map of the mask
 // left behind; a separate instantiation, so that the kernel of a caller who wants neither carries
 // none of that code (it measured 1.5 % on the headline workload even when switched off at run time).
-template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int HDIM, bool BYTEMASK = false, bool BYPRODUCTS = false>
+// PAIRS (with BYTEMASK, head dims up to 64, N a multiple of 128, no by-products): the mask bytes of
+// TWO key tiles are requested at once, every second visit: 128 bytes per row, i.e. whole cache lines
+// where one tile's 64 bytes are half of one.  From 640 keys on the forward from the boolean mask
+// measured 2 to 4 % faster this way on random masks and 7 % on the block-structured workload; below
+// (few visits, of which the first then waits for twice the bytes) it is 2 to 3 % slower and the
+// launcher leaves it off.
+template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int HDIM, bool BYTEMASK = false, bool BYPRODUCTS = false,
+          bool PAIRS = false>
 __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel(const AttnArgs a)
 {
+    static_assert(!PAIRS || (BYTEMASK && !BYPRODUCTS && HDIM <= 64), "PAIRS: byte mask, two byte slots, no by-products");
     using E = Elem<BF16>;
     constexpr int NH = HDIM == 128 ? 2 : 1;       // 64-column tiles per matrix
     constexpr int KS = HDIM / 16;                 // MFMA steps of the QK^T chain
@@ -218,6 +226,23 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
             async_copy_b32_at<OFF_MASK + SLOT * MASK_SLOT>(mask_dst, mb + 2 * x, voff);
         }
     };
+    // PAIRS: four copies per wave and pair of tiles; lane i of copy j fills (row 8j + i/8, position i%8)
+    // from the row's chunk (i%8) ^ ((row >> 1) & 7).  (row >> 1) & 7 is (i/8 >> 1) for j = 0, 2 and that
+    // plus 4 for j = 1, 3: one lane offset and the same with chunk bit 2 flipped (N is a multiple of
+    // 128, so the low seven bits of the offset are the chunk alone).
+    uint32_t pair_voff = 0u;
+    if constexpr (PAIRS) {
+        const int row = lane >> 3;
+        pair_voff = (uint32_t)(qt * BM + wave * 32 + row) * (uint32_t)N + (uint32_t)(((lane & 7) ^ (row >> 1)) << 4);
+    }
+    auto issue_mask_pair = [&](int p) __attribute__((always_inline)) {      // bytes of tiles 2p and 2p + 1
+        const uint8_t *src = reinterpret_cast<const uint8_t *>(mb) + (size_t)p * (2 * BN);
+        const uint32_t dst = lds0 + wave * 4096;
+        async_copy_b128_at<OFF_MASK>(dst, src, pair_voff);
+        async_copy_b128_at<OFF_MASK + 1024>(dst, src + (size_t)8 * N, pair_voff ^ 64u);
+        async_copy_b128_at<OFF_MASK + 2048>(dst, src + (size_t)16 * N, pair_voff);
+        async_copy_b128_at<OFF_MASK + 3072>(dst, src + (size_t)24 * N, pair_voff ^ 64u);
+    };
     // BYTEMASK: where this lane's row of packed words goes, if the caller wants them ([Bm, Hm, N, nw]
     // like the mask; a mask shared between batch entries / heads is written by the first of them)
     const int qrow = qt * BM + wave * 32 + l32;
@@ -245,12 +270,22 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     }
     const uint32_t maddr = BYTEMASK ? lds0 + OFF_MASK + wave * 2048 + l32 * 64 : lds0 + OFF_MASK + wave * 256 + l32 * 8;
     const int msw = (l32 >> 2) & 3;
-    auto mask_words = [&](int x, int slot) __attribute__((always_inline)) -> u32x2 {
+    // PAIRS: a wave's bytes of a pair of tiles are 32 rows of 128 bytes in the 4 KiB that its two byte
+    // slots occupy otherwise; the 16-byte chunks of a row are swizzled like K's (position ^ ((row >> 1)
+    // & 7), applied on the global side), which keeps the reads below free of bank conflicts.
+    // `pair_half` (0 or 1) says which tile of the pair; -1: the ordinary slots.
+    const uint32_t pair_base = lds0 + OFF_MASK + wave * 4096 + l32 * 128;
+    const int psw = (l32 >> 1) & 7;
+    auto mask_words = [&](int x, int slot, int pair_half = -1) __attribute__((always_inline)) -> u32x2 {
         u32x2 w;
         if constexpr (BYTEMASK) {
             // this lane: the 32 bytes of row l32 for keys 32hh .. 32hh+31 -> one word
-            const u32x4 d0 = lds_read_b128(maddr + slot * MASK_SLOT + (((2 * hh) ^ msw) << 4));
-            const u32x4 d1 = lds_read_b128(maddr + slot * MASK_SLOT + (((2 * hh + 1) ^ msw) << 4));
+            const uint32_t a0 = !PAIRS || pair_half < 0 ? maddr + slot * MASK_SLOT + (((2 * hh) ^ msw) << 4)
+                                                        : pair_base + (((4 * pair_half + 2 * hh) ^ psw) << 4);
+            const uint32_t a1 = !PAIRS || pair_half < 0 ? maddr + slot * MASK_SLOT + (((2 * hh + 1) ^ msw) << 4)
+                                                        : pair_base + (((4 * pair_half + 2 * hh + 1) ^ psw) << 4);
+            const u32x4 d0 = lds_read_b128(a0);
+            const u32x4 d1 = lds_read_b128(a1);
             // a byte counts as "attend" when it is non-zero, as in the packer: nz() leaves 0x80 in
             // every non-zero byte, the dot products weigh those with 1, 2, 4 .. 128 (times 128)
             auto nz = [](uint32_t x) -> uint32_t { return (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u; };
@@ -469,15 +504,21 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
     };
     const int t_first = next_tile();
     if (t_first < T) {
-        issue_kv(t_first, integral_constant<int, 0>{});
-        issue_mask(t_first, integral_constant<int, 0>{});
+        if constexpr (PAIRS) {          // the first pair's bytes before K/V: the walk below counts on that order
+            issue_mask_pair(0);
+            issue_kv(t_first, integral_constant<int, 0>{});
+        } else {
+            issue_kv(t_first, integral_constant<int, 0>{});
+            issue_mask(t_first, integral_constant<int, 0>{});
+        }
     }
     // small LDS table for the mask: entry n (16 B) holds four floats, float j = (bit j of n) ? 0 : -inf
     if (tid < 64)
         reinterpret_cast<float *>(smem + OFF_LUT)[tid] = (((tid >> 2) >> (tid & 3)) & 1) ? 0.f : -__builtin_inff();
     const bool even_progress = NH == 1 && (int)blockIdx.x >= a.tail_start;   // three work-groups per CU
     if (even_progress && n_visits >= 4) __builtin_amdgcn_s_setprio(3);
-    if (t_first < T) wait_vmcnt<C::COPIES>();     // q has landed; the copies of the first tile may still be in flight
+    if (PAIRS) wait_vmcnt<8>();                   // q has landed; 4 mask and 4 K/V copies may still be in flight
+    else if (t_first < T) wait_vmcnt<C::COPIES>();     // q has landed; the copies of the first tile may still be in flight
     else wait_vmcnt<0>();
     // ---- Q^T as MFMA B operands, scaled by scale*log2(e)/post_mul:
     //      lane holds query row l32, d = 16*s + 8*hh .. +7
@@ -688,6 +729,37 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         }
         compute_tile(w2, (uint32_t)(SLOT * STAGE_BYTES));
     };
+    if constexpr (PAIRS) {
+        // Every tile is visited (there is no tile map with a boolean mask) and their number is even.
+        // Copies in flight, oldest first, at the top of an even visit t: the bytes of the pair
+        // (t, t + 1), then K/V of t; after its barrier K/V of t + 1 and then the bytes of the next
+        // pair are requested, and the odd visit requests K/V of t + 2 after its barrier: the bytes of
+        // a pair are always followed by exactly four younger copies when they are needed.
+        auto progress = [&]() __attribute__((always_inline)) {
+            if (even_progress) {
+                if (visits == n_visits / 4) __builtin_amdgcn_s_setprio(2);
+                else if (visits == n_visits / 2) __builtin_amdgcn_s_setprio(1);
+                else if (visits == (3 * n_visits) / 4) __builtin_amdgcn_s_setprio(0);
+            }
+            ++visits;
+        };
+        for (int t = 0; t < T; t += 2) {
+            progress();
+            wait_vmcnt<4>();                                  // this wave's bytes of the pair have landed
+            const u32x2 w_even = mask_words(t, 0, 0);
+            const u32x2 w_odd = mask_words(t + 1, 0, 1);
+            wait_vmcnt<0>();                                  // K/V of tile t
+            __syncthreads();
+            issue_kv(t + 1, integral_constant<int, 1>{});
+            if (t + 2 < T) issue_mask_pair((t >> 1) + 1);     // the words above are in registers: the bytes may go
+            compute_tile(w_even, 0u);
+            progress();
+            if (t + 2 < T) wait_vmcnt<4>(); else wait_vmcnt<0>();   // K/V of tile t + 1 (the next pair's bytes may be on their way)
+            __syncthreads();
+            if (t + 2 < T) issue_kv(t + 2, integral_constant<int, 0>{});
+            compute_tile(w_odd, (uint32_t)STAGE_BYTES);
+        }
+    } else
     for (int t = t_first; t < T;) {
         const int tn = next_tile();
         visit(t, tn, integral_constant<int, 0>{});
@@ -745,7 +817,9 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         if (a.lse != nullptr && hh == 0) {
             // log2 of the row's sum of exp(scale * score) is pm * r + log2(l)
             a.lse[(size_t)bh * N + qrow] =
-                (l_tot > 0.f) ? (pm * ref) * 0.6931471805599453f + __builtin_logf(l_tot) : -__builtin_inff();
+                (l_tot > 0.f) ? __builtin_fmaf(pm * ref, 0.6931471805599453f, __builtin_logf(l_tot)) : -__builtin_inff();
+            // (an explicit fma: left to the compiler, the sum was contracted in some instantiations of
+            // this kernel and not in others, and their lse differed in the last bit)
         }
     }
 }
@@ -813,13 +887,29 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     case 14: kernel = attn_fwd_kernel<true, true, false, HDIM, true, true>; break;     \
     default: kernel = attn_fwd_kernel<true, true, true, HDIM, true, true>; break;      \
     }
+#define SMA_FWD_PAIRS_VARIANTS(HDIM)                                                    \
+    switch (variant) {                                                                 \
+    case 0: kernel = attn_fwd_kernel<false, false, false, HDIM, true, false, true>; break;   \
+    case 1: kernel = attn_fwd_kernel<false, false, true, HDIM, true, false, true>; break;    \
+    case 2: kernel = attn_fwd_kernel<false, true, false, HDIM, true, false, true>; break;    \
+    case 3: kernel = attn_fwd_kernel<false, true, true, HDIM, true, false, true>; break;     \
+    case 4: kernel = attn_fwd_kernel<true, false, false, HDIM, true, false, true>; break;    \
+    case 5: kernel = attn_fwd_kernel<true, false, true, HDIM, true, false, true>; break;     \
+    case 6: kernel = attn_fwd_kernel<true, true, false, HDIM, true, false, true>; break;     \
+    default: kernel = attn_fwd_kernel<true, true, true, HDIM, true, false, true>; break;     \
+    }
     const bool byproducts = a.mask_out != nullptr || a.map_out != nullptr;
-    if (a.byte_mask) {
+    // two tiles' mask bytes per request: see PAIRS at the kernel
+    const bool pairs = a.byte_mask && !byproducts && D <= 64 && a.N >= 640 && a.N % (2 * BN) == 0;
+    if (pairs) {
+        if (D == 32) { SMA_FWD_PAIRS_VARIANTS(32) } else { SMA_FWD_PAIRS_VARIANTS(64) }
+    } else if (a.byte_mask) {
         if (a.N < 16) return hipErrorInvalidValue;          // a row holds at least one 16-byte copy (checked by the C-ABI layer)
         if (D == 32) { SMA_FWD_BYTEMASK_VARIANTS(32) } else if (D == 64) { SMA_FWD_BYTEMASK_VARIANTS(64) } else { SMA_FWD_BYTEMASK_VARIANTS(128) }
     } else if (D == 32) { SMA_FWD_VARIANTS(32) } else if (D == 64) { SMA_FWD_VARIANTS(64) } else { SMA_FWD_VARIANTS(128) }
 #undef SMA_FWD_VARIANTS
 #undef SMA_FWD_BYTEMASK_VARIANTS
+#undef SMA_FWD_PAIRS_VARIANTS
     hipLaunchKernelGGL(kernel, grid, block, 0, stream, a);
     return hipGetLastError();
 }

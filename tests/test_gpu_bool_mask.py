@@ -98,6 +98,52 @@ def test_scales_many_heads_and_long_rows(dev):
     torch.cuda.synchronize()
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("D", [32, 64])
+@pytest.mark.parametrize("N", [640, 768, 1152, 2048])
+def test_two_tiles_of_mask_bytes_per_request(dev, dtype, D, N):
+    """From 640 keys on, with N a multiple of 128 and head dims up to 64, the kernel requests the mask
+    bytes of two key tiles at once (whole 128-byte lines).  Same arithmetic, so out and lse must be
+    those of pack + attention bit for bit: with a mask per head, with one mask for all, with bytes
+    other than 0 and 1, at an odd byte address, for a scale that takes the post-multiplied exponent,
+    and through strided q, k, v, out.  (N = 1152 has an odd number of pairs' worth of 64-key tiles
+    beyond a power of two; 2048 runs several rounds of work-groups.)"""
+    B, H = 2, 3
+    q, k, v, mask = _inputs(B, H, N, D, dtype, 900 + N + D, keep=0.2)
+    mask[1, 0, 7, :] = False                       # a row that keeps nothing
+    mask[0, 2, :, 64:192] = False                  # a pair of key tiles nobody in this head keeps
+    qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
+    packed = _capi.pack_mask(md)
+    for scale in (1.0, None):
+        want, want_lse = _capi.attn_fwd(qd, kd, vd, packed, scale=scale, want_lse=True)
+        got, lse = _capi.attn_fwd_bool_mask(qd, kd, vd, md, scale=scale, want_lse=True)
+        torch.cuda.synchronize()
+        assert torch.equal(got, want) and torch.equal(lse, want_lse), scale
+    ref = O.sparse_attention_ref(q.float(), k.float(), v.float(), mask)
+    assert torch.allclose(got.float().cpu(), ref, atol=1e-2, rtol=2e-2)
+    assert (got[1, 0, 7] == 0).all() and lse[1, 0, 7].item() == -math.inf
+    # one mask for every batch entry and head
+    one = mask[:1, :1].contiguous().to(dev)
+    want = _capi.attn_fwd(qd, kd, vd, _capi.pack_mask(one.expand(B, H, N, N).contiguous()))
+    assert torch.equal(_capi.attn_fwd_bool_mask(qd, kd, vd, one), want)
+    # bytes other than 0 and 1, at an odd address
+    raw = torch.zeros(3 + mask.numel(), dtype=torch.uint8, device=dev)
+    g = torch.Generator().manual_seed(N)
+    values = torch.randint(1, 256, mask.shape, generator=g, dtype=torch.int32).to(torch.uint8)
+    raw[3:].view(B, H, N, N).copy_((values * mask).to(dev))
+    odd = raw[3:].view(B, H, N, N).view(torch.bool)
+    assert odd.data_ptr() % 16 == (raw.data_ptr() + 3) % 16
+    want, want_lse = _capi.attn_fwd(qd, kd, vd, packed, want_lse=True)
+    got, lse = _capi.attn_fwd_bool_mask(qd, kd, vd, odd, want_lse=True)
+    assert torch.equal(got, want) and torch.equal(lse, want_lse)
+    # strided q, k, v, out ([B,N,H,D] buffers)
+    qs, ks, vs = (t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) for t in (qd, kd, vd))
+    out_view = torch.empty(B, N, H, D, dtype=dtype, device=dev).permute(0, 2, 1, 3)
+    got = _capi.attn_fwd_bool_mask_strided(qs, ks, vs, md, out=out_view)
+    torch.cuda.synchronize()
+    assert torch.equal((got[0] if isinstance(got, tuple) else got).contiguous(), want)
+
+
 def test_limits_are_reported(dev):
     q, k, v, mask = _inputs(1, 1, 15, 64, torch.float16, 70)                   # a row shorter than one 16-byte copy
     qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))

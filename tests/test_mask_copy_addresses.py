@@ -7,7 +7,8 @@ so that for every sequence length
     after the last byte is read),
   * the chunk a lane converts holds the 16 columns it stands for, or, for the chunk that contains
     the row's end, those columns after the right shift the kernel applies.
-Second, the packer's row loads (csrc/pack_mask.hip), further down."""
+Second, the same forward when it requests two tiles' bytes at once; third, the packer's row loads
+(csrc/pack_mask.hip), further down."""
 import numpy as np
 import pytest
 
@@ -56,6 +57,48 @@ def test_every_length_up_to_1100():
 @pytest.mark.parametrize("N", [2047, 4095, 8191, 46340])
 def test_long_rows(N):
     _check(N)
+
+
+def _check_pairs(N):
+    """The same forward when it requests the bytes of two key tiles at once (attn_fwd.hip,
+    issue_mask_pair / mask_words with pair_half; N a multiple of 128): restated for every lane of
+    every wave and every pair, so that each 16-byte copy lies inside the row it is meant for, every
+    chunk of the pair lands exactly once in the wave's 4 KiB, and the two chunks a lane reads for a
+    tile are the 32 columns it stands for."""
+    assert N % 128 == 0
+    qtiles = N // BM
+    lane = np.arange(64)
+    for qt in {0, qtiles - 1}:
+        for wave in range(4):
+            for p in {0, N // 128 - 1}:
+                lds = np.full((32, 8), -1, dtype=np.int64)        # [row][position] -> first column held
+                r = lane >> 3
+                voff0 = (qt * BM + wave * 32 + r).astype(np.int64) * N + (((lane & 7) ^ (r >> 1)) << 4)
+                for j in range(4):
+                    voff = voff0 ^ 64 if j & 1 else voff0
+                    assert (voff >= 0).all() and (voff < 2**32).all()
+                    addr = p * 128 + 8 * j * N + voff
+                    row = 8 * j + r
+                    grow = qt * BM + wave * 32 + row
+                    col0 = addr - grow.astype(np.int64) * N
+                    assert (col0 >= p * 128).all() and (col0 + 16 <= (p + 1) * 128).all(), (N, p, j)
+                    assert (grow < N).all() and (addr + 16 <= N * N).all()
+                    dst = j * 1024 + lane * 16                      # byte in the wave's 4 KiB
+                    assert ((dst >> 7) == row).all()
+                    lds[row, (dst >> 4) & 7] = col0
+                assert (lds >= 0).all()
+                for half in range(2):                               # which tile of the pair
+                    for l32 in range(32):
+                        for hh in range(2):
+                            psw = (l32 >> 1) & 7
+                            for k in range(2):
+                                pos = (4 * half + 2 * hh + k) ^ psw
+                                assert lds[l32, pos] == p * 128 + half * 64 + 32 * hh + 16 * k, (N, p, half, l32, hh, k)
+
+
+def test_pairs_of_tiles():
+    for N in (128, 640, 768, 1024, 2048, 4096, 46336):
+        _check_pairs(N)
 
 
 def _check_packer_row(N, lanes_per_row=64):
