@@ -106,7 +106,7 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_
 // BYPRODUCTS (with BYTEMASK): the caller wants the packed words and / or the tile map of the mask
 // left behind; a separate instantiation, so that the kernel of a caller who wants neither carries
 // none of that code (it measured 1.5 % on the headline workload even when switched off at run time).
-// PAIRS (with BYTEMASK, head dims up to 64, N a multiple of 128, no by-products): the mask bytes of
+// PAIRS (with BYTEMASK, head dims up to 64, N a multiple of 128): the mask bytes of
 // TWO key tiles are requested at once, every second visit: 128 bytes per row, i.e. whole cache lines
 // where one tile's 64 bytes are half of one.  From 640 keys on the forward from the boolean mask
 // measured 2 to 4 % faster this way on random masks and 7 % on the block-structured workload; below
@@ -116,7 +116,7 @@ template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int HDIM, bool BYTEMASK = f
           bool PAIRS = false>
 __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel(const AttnArgs a)
 {
-    static_assert(!PAIRS || (BYTEMASK && !BYPRODUCTS && HDIM <= 64), "PAIRS: byte mask, two byte slots, no by-products");
+    static_assert(!PAIRS || (BYTEMASK && HDIM <= 64), "PAIRS: byte mask, two byte slots");
     using E = Elem<BF16>;
     constexpr int NH = HDIM == 128 ? 2 : 1;       // 64-column tiles per matrix
     constexpr int KS = HDIM / 16;                 // MFMA steps of the QK^T chain
@@ -734,7 +734,9 @@ __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel
         // Copies in flight, oldest first, at the top of an even visit t: the bytes of the pair
         // (t, t + 1), then K/V of t; after its barrier K/V of t + 1 and then the bytes of the next
         // pair are requested, and the odd visit requests K/V of t + 2 after its barrier: the bytes of
-        // a pair are always followed by exactly four younger copies when they are needed.
+        // a pair are always followed by exactly four younger copies when they are needed.  (The stores
+        // of the by-products, when asked for, only add to the count: copies complete in the order of
+        // their requests, so "at most four outstanding" still means that all older copies are in.)
         auto progress = [&]() __attribute__((always_inline)) {
             if (even_progress) {
                 if (visits == n_visits / 4) __builtin_amdgcn_s_setprio(2);
@@ -888,7 +890,7 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     default: kernel = attn_fwd_kernel<true, true, true, HDIM, true, true>; break;      \
     }
 #define SMA_FWD_PAIRS_VARIANTS(HDIM)                                                    \
-    switch (variant) {                                                                 \
+    switch (variant | (byproducts ? 8 : 0)) {                                          \
     case 0: kernel = attn_fwd_kernel<false, false, false, HDIM, true, false, true>; break;   \
     case 1: kernel = attn_fwd_kernel<false, false, true, HDIM, true, false, true>; break;    \
     case 2: kernel = attn_fwd_kernel<false, true, false, HDIM, true, false, true>; break;    \
@@ -896,11 +898,19 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     case 4: kernel = attn_fwd_kernel<true, false, false, HDIM, true, false, true>; break;    \
     case 5: kernel = attn_fwd_kernel<true, false, true, HDIM, true, false, true>; break;     \
     case 6: kernel = attn_fwd_kernel<true, true, false, HDIM, true, false, true>; break;     \
-    default: kernel = attn_fwd_kernel<true, true, true, HDIM, true, false, true>; break;     \
+    case 7: kernel = attn_fwd_kernel<true, true, true, HDIM, true, false, true>; break;      \
+    case 8: kernel = attn_fwd_kernel<false, false, false, HDIM, true, true, true>; break;    \
+    case 9: kernel = attn_fwd_kernel<false, false, true, HDIM, true, true, true>; break;     \
+    case 10: kernel = attn_fwd_kernel<false, true, false, HDIM, true, true, true>; break;    \
+    case 11: kernel = attn_fwd_kernel<false, true, true, HDIM, true, true, true>; break;     \
+    case 12: kernel = attn_fwd_kernel<true, false, false, HDIM, true, true, true>; break;    \
+    case 13: kernel = attn_fwd_kernel<true, false, true, HDIM, true, true, true>; break;     \
+    case 14: kernel = attn_fwd_kernel<true, true, false, HDIM, true, true, true>; break;     \
+    default: kernel = attn_fwd_kernel<true, true, true, HDIM, true, true, true>; break;      \
     }
     const bool byproducts = a.mask_out != nullptr || a.map_out != nullptr;
     // two tiles' mask bytes per request: see PAIRS at the kernel
-    const bool pairs = a.byte_mask && !byproducts && D <= 64 && a.N >= 640 && a.N % (2 * BN) == 0;
+    const bool pairs = a.byte_mask && D <= 64 && a.N >= 640 && a.N % (2 * BN) == 0;
     if (pairs) {
         if (D == 32) { SMA_FWD_PAIRS_VARIANTS(32) } else { SMA_FWD_PAIRS_VARIANTS(64) }
     } else if (a.byte_mask) {

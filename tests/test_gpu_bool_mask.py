@@ -136,6 +136,12 @@ def test_two_tiles_of_mask_bytes_per_request(dev, dtype, D, N):
     want, want_lse = _capi.attn_fwd(qd, kd, vd, packed, want_lse=True)
     got, lse = _capi.attn_fwd_bool_mask(qd, kd, vd, odd, want_lse=True)
     assert torch.equal(got, want) and torch.equal(lse, want_lse)
+    # with the by-products asked for (what the training forward does): words and tile map as the packer makes them
+    got, lse, words, tmap = _capi.attn_fwd_bool_mask(qd, kd, vd, md, want_lse=True, want_packed=True, want_map=True)
+    want_words, want_map = _capi.pack_mask_map(md)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want) and torch.equal(lse, want_lse)
+    assert torch.equal(words, want_words) and torch.equal(tmap, want_map)
     # strided q, k, v, out ([B,N,H,D] buffers)
     qs, ks, vs = (t.permute(0, 2, 1, 3).contiguous().permute(0, 2, 1, 3) for t in (qd, kd, vd))
     out_view = torch.empty(B, N, H, D, dtype=dtype, device=dev).permute(0, 2, 1, 3)
@@ -173,7 +179,7 @@ def test_mask_at_any_byte_address(dev, offset):
 
 
 @pytest.mark.parametrize("shape", ["BH", "11", "B1", "1H"])
-@pytest.mark.parametrize("N", [16, 35, 80, 128, 250, 400, 1001, 1008])
+@pytest.mark.parametrize("N", [16, 35, 80, 128, 250, 400, 640, 1001, 1008, 1152])
 def test_packed_words_are_left_behind(dev, N, shape):
     """packed_out receives exactly what sma_pack_mask writes (every word, pad bits zero), so that a
     backward can follow without a packing pass; shared masks are written once."""

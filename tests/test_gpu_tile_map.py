@@ -58,7 +58,7 @@ def test_tile_map_matches_the_oracle(dev, N):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("D", [32, 64, 128])
-@pytest.mark.parametrize("N", [16, 17, 63, 64, 65, 127, 128, 129, 200, 256, 333, 512, 1000])
+@pytest.mark.parametrize("N", [16, 17, 63, 64, 65, 127, 128, 129, 200, 256, 333, 512, 640, 1000, 1152])
 def test_forward_from_bool_mask_leaves_the_tile_map(dev, N, D, dtype):
     """The map that comes out of the one-launch forward equals the oracle's, with and without the
     packed words being asked for, and asking for it changes neither the output nor the lse."""
