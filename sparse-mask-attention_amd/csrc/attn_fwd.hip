@@ -108,10 +108,12 @@ template <int N> __device__ __forceinline__ void wait_vmcnt() { asm volatile("s_
 // none of that code (it measured 1.5 % on the headline workload even when switched off at run time).
 // PAIRS (with BYTEMASK, head dims up to 64, N a multiple of 128): the mask bytes of
 // TWO key tiles are requested at once, every second visit: 128 bytes per row, i.e. whole cache lines
-// where one tile's 64 bytes are half of one.  From 640 keys on the forward from the boolean mask
-// measured 2 to 4 % faster this way on random masks and 7 % on the block-structured workload; below
-// (few visits, of which the first then waits for twice the bytes) it is 2 to 3 % slower and the
-// launcher leaves it off.
+// where one tile's 64 bytes are half of one.  The forward from the boolean mask measured 1 to 5 %
+// faster this way on random masks of every length tried (128 to 2048) and 7 % on the
+// block-structured workload -- except where the whole grid is one round of work-groups that run in
+// step (the even-progress case of the launcher, e.g. the headline shape): there the first visit,
+// which waits for twice the bytes, is not hidden behind other work-groups' work, it measured 1 to 4 %
+// slower, and the launcher leaves it off.
 template <bool BF16, bool POSTMUL, bool PACKED_ROWS, int HDIM, bool BYTEMASK = false, bool BYPRODUCTS = false,
           bool PAIRS = false>
 __global__ __launch_bounds__(NTHREADS, HDIM == 128 ? 2 : 3) void attn_fwd_kernel(const AttnArgs a)
@@ -909,8 +911,9 @@ hipError_t launch_attn_fwd(const AttnArgs &args, bool bf16, hipStream_t stream)
     default: kernel = attn_fwd_kernel<true, true, true, HDIM, true, true, true>; break;      \
     }
     const bool byproducts = a.mask_out != nullptr || a.map_out != nullptr;
-    // two tiles' mask bytes per request: see PAIRS at the kernel
-    const bool pairs = a.byte_mask && D <= 64 && a.N >= 640 && a.N % (2 * BN) == 0;
+    // two tiles' mask bytes per request (see PAIRS at the kernel), unless the grid is the single round
+    // of work-groups in step for which tail_start was set to 0 above
+    const bool pairs = a.byte_mask && D <= 64 && a.N % (2 * BN) == 0 && a.tail_start != 0;
     if (pairs) {
         if (D == 32) { SMA_FWD_PAIRS_VARIANTS(32) } else { SMA_FWD_PAIRS_VARIANTS(64) }
     } else if (a.byte_mask) {

@@ -100,10 +100,12 @@ def test_scales_many_heads_and_long_rows(dev):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("D", [32, 64])
-@pytest.mark.parametrize("N", [640, 768, 1152, 2048])
+@pytest.mark.parametrize("N", [128, 384, 640, 1152, 2048])
 def test_two_tiles_of_mask_bytes_per_request(dev, dtype, D, N):
-    """From 640 keys on, with N a multiple of 128 and head dims up to 64, the kernel requests the mask
-    bytes of two key tiles at once (whole 128-byte lines).  Same arithmetic, so out and lse must be
+    """With N a multiple of 128 and head dims up to 64 the kernel requests the mask bytes of two key
+    tiles at once (whole 128-byte lines), unless the grid is a single round of work-groups in step
+    (512 < B*H*ceil(N/128) <= 768 on this part, e.g. the headline workload, which
+    test_benchmark_workloads_at_full_size runs).  Same arithmetic, so out and lse must be
     those of pack + attention bit for bit: with a mask per head, with one mask for all, with bytes
     other than 0 and 1, at an odd byte address, for a scale that takes the post-multiplied exponent,
     and through strided q, k, v, out.  (N = 1152 has an odd number of pairs' worth of 64-key tiles
@@ -111,7 +113,7 @@ def test_two_tiles_of_mask_bytes_per_request(dev, dtype, D, N):
     B, H = 2, 3
     q, k, v, mask = _inputs(B, H, N, D, dtype, 900 + N + D, keep=0.2)
     mask[1, 0, 7, :] = False                       # a row that keeps nothing
-    mask[0, 2, :, 64:192] = False                  # a pair of key tiles nobody in this head keeps
+    mask[0, 2, :, 0:128] = False                   # a pair of key tiles nobody in this head keeps
     qd, kd, vd, md = (t.to(dev) for t in (q, k, v, mask))
     packed = _capi.pack_mask(md)
     for scale in (1.0, None):
